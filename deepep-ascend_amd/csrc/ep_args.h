@@ -1,0 +1,103 @@
+// Kernel argument blocks shared by the device code object (ep_kernels.hip) and the host
+// runtime (ep_runtime.cpp).  Every kernel takes exactly one of these structs by value, so a
+// launch through hipModuleLaunchKernel marshals a single parameter.
+#pragma once
+#include <stdint.h>
+
+#define EP_MAX_RANKS 256          // reference: common/compiled.hpp:35
+#define EP_MAX_EXPERTS 2048       // reference: common/compiled.hpp:36
+#define EP_MAX_TOPK 32            // reference: csrc/kernels/ep/combine.hpp:85
+#define EP_TOKENS_PER_BLOCK 128   // tokens owned by one layout workgroup
+#define EP_LAYOUT_THREADS 256
+#define EP_SCAN_THREADS 1024
+#define EP_ROW_THREADS 256        // 4 waves, one row per wave
+#define EP_ROWS_PER_BLOCK 4
+#define EP_PAD_BLOCKS_PER_EXPERT 4
+
+// Host-visible count page (pinned, mapped).  Written once per non-cached dispatch.
+//   [0] ready sequence number (written last, release at system scope)
+//   [1] number of received tokens   [2] number of expanded tokens (aligned)
+//   [16 .. 16+R)                 received tokens per source rank
+//   [16+EP_MAX_RANKS .. +El)     aligned received tokens per local expert
+#define EP_HOST_RANK_OFF 16
+#define EP_HOST_EXPERT_OFF (16 + EP_MAX_RANKS)
+#define EP_HOST_PAGE_INTS (16 + EP_MAX_RANKS + EP_MAX_EXPERTS)
+
+struct EpLayoutArgs {
+    const int64_t* topk_idx;      // [T, K]
+    int num_tokens, num_topk, num_experts, num_ranks;
+    int rank_idx, expert_alignment, max_tokens, experts_per_rank;
+    int num_blocks;               // ceil(T / EP_TOKENS_PER_BLOCK), at least 1
+    int seq;                      // value the host waits for in host_page[0]
+    int notify_host;              // do_cpu_sync
+    int pad0;
+    // scratch (device)
+    int* blk_expert_cnt;          // [num_blocks, E]   counts, then exclusive prefix over blocks
+    int* blk_rank_cnt;            // [num_blocks, R]   master counts, then exclusive prefix
+    int* expert_total;            // [E]
+    int* rank_total;              // [R]
+    int* slot_map;                // [T, K]  expanded slot of (t, j) if its expert is local, else -1
+    int* recv_tok;                // [max_tokens]  receive-stream row -> local token index
+    // handle tensors (device)
+    int* dst_buffer_slot_idx;     // [T, K]
+    int* dst_gsge_idx;            // [T, K]
+    int* psum_rank;               // [R]
+    int* psum_expert;             // [El]
+    int* unaligned_expert;        // [El]
+    int* cumulative_stats;        // [El] or null
+    int* host_page;               // device view of the mapped host page
+};
+
+// One receive-stream row per wave: copy (or quantise) it into every expanded slot it owns.
+struct EpScatterArgs {
+    const void* x;                // [T, hidden] rows: BF16, or FP8 bytes when prequantised
+    const void* sf;               // input scale factors (prequantised FP8) or null
+    const float* topk_weights;    // [T, K] or null
+    const int* slot_map;          // [T, K]   (non-cached)
+    const int* recv_tok;          // [N]      (non-cached)
+    const int* num_recv_ptr;      // device scalar: psum_rank[R-1]
+    int* recv_src_metadata;       // [N, K+2]  written (non-cached) / read (cached)
+    void* recv_x;                 // [N_exp, hidden] out
+    void* recv_sf;                // out or null
+    float* recv_topk_weights;     // [N_exp] out or null
+    const int* psum_expert;       // [El]  (padding ranges)
+    int64_t x_row_bytes;          // bytes per source row
+    int64_t out_row_bytes;        // bytes per output row
+    int64_t sf_token_stride_bytes, sf_pack_stride_bytes;   // input SF strides
+    int64_t out_sf_row_bytes;
+    int hidden;                   // channels per row
+    int num_topk, num_rows_bound;     // grid covers rows [0, num_rows_bound)
+    int rank_idx, max_tokens;
+    int cached;                   // slots come from recv_src_metadata
+    int num_sf_packs;             // 2-byte packs per row (prequantised) ; fused: hidden/128 floats
+    int num_local_experts, expert_alignment;
+    int zero_padding;
+    int num_row_blocks;           // blocks [0, num_row_blocks) copy rows, the rest zero padding
+    int num_tokens;               // T: bound of the token indices a row may name
+};
+
+// Fused single-partition combine: one receive-stream row per wave.
+struct EpCombineArgs {
+    const void* y;                // [N_exp, hidden] BF16 expert outputs
+    const float* expanded_weights;// [N_exp] or null
+    const void* bias_0;           // [T, hidden] BF16 or null
+    const void* bias_1;
+    const int* recv_src_metadata; // [N, K+2]
+    const int* num_recv_ptr;      // device scalar
+    const int64_t* topk_idx;      // [T, K]
+    void* combined_x;             // [T, hidden] BF16 out
+    float* combined_topk_weights; // [T, K] out or null
+    int hidden, num_topk, num_tokens, num_rows_bound;
+    int rank_idx, max_tokens;
+    int weighted;                 // opt-in: multiply by the gate weight before summing
+    int num_row_blocks;           // blocks [0, num_row_blocks) reduce rows, the rest handle unrouted tokens
+    int num_experts, pad0;
+};
+
+// Hardware vs integer e4m3fn conversion over fp32 bit patterns [first, first+count).
+struct EpFp8TestArgs {
+    unsigned long long first, count;
+    unsigned long long* out;      // [0] mismatches, [1] first mismatching pattern
+    float limit;                  // only |x| <= limit is compared (NaN patterns are skipped)
+    int pad;
+};

@@ -1,0 +1,658 @@
+// Device code object for the EP dispatch/combine path on gfx950 (wave64).  Built ahead of time with
+// `hipcc --genco` and launched by the host runtime through hipModuleLaunchKernel.
+//
+// Kernels (all HBM-bound, no MFMA):
+//   ep_layout_count / ep_layout_scan / ep_layout_assign   stable counting sort of the (token, slot)
+//       entries by destination partition and by local expert -> every handle tensor
+//   ep_scatter_copy / ep_scatter_quant                     receive-stream row -> its expanded slots
+//   ep_combine_k<K> / ep_combine_generic                   K-way gather + fp32 reduce back to token order
+//   ep_fp8_selftest                                        hardware vs integer e4m3fn conversion
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ep_args.h"
+#include "ep_fp8.h"
+
+#define WAVE 64
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+__device__ __forceinline__ int align_up(int x, int a) { return (x + a - 1) / a * a; }
+
+__device__ __forceinline__ int readlane(int v, int l) { return __builtin_amdgcn_readlane(v, l); }
+
+// Lanes of the wave holding the same key.  Every lane must call it; `key` < 2^nbits.
+__device__ __forceinline__ uint64_t match_any(int key, int nbits) {
+    uint64_t peers = ~0ull;
+    for (int b = 0; b < nbits; ++b) {
+        const bool bit = (key >> b) & 1;
+        const uint64_t ones = __ballot(bit);
+        peers &= bit ? ones : ~ones;
+    }
+    return peers;
+}
+
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int off = 1; off < WAVE; off <<= 1) {
+        const int o = __shfl_up(v, off, WAVE);
+        if (lane >= off) v += o;
+    }
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Layout pass A: per-block histograms of expert ids and of destination-partition masters.
+// Reference semantics: impls/ep/dispatch.hpp:166-194 (expert histogram, dedup by partition).
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s_key, short* s_rk) {
+    const int K = a.num_topk;
+    const int n = EP_TOKENS_PER_BLOCK * K;
+    const int64_t base = (int64_t)blockIdx.x * n;
+    const int64_t total = (int64_t)a.num_tokens * K;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        int e = -1;
+        if (base + i < total) {
+            const int64_t v = a.topk_idx[base + i];
+            e = (v >= 0 && v < a.num_experts) ? (int)v : -1;
+        }
+        s_key[i] = (short)e;
+        s_rk[i] = (short)(e < 0 ? -1 : e / a.experts_per_rank);
+    }
+}
+
+// Destination partition of entry idx if it is the last slot of its token going there, else -1
+// (the "master" of common/simt.hpp:24-34).
+__device__ __forceinline__ int master_rank(const short* s_rk, int idx, int K) {
+    const int r = s_rk[idx];
+    if (r < 0) return -1;
+    const int j = idx % K;
+    for (int jj = j + 1; jj < K; ++jj)
+        if (s_rk[idx - j + jj] == r) return -1;
+    return r;
+}
+
+extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(EpLayoutArgs a) {
+    extern __shared__ int smem[];
+    const int E = a.num_experts, R = a.num_ranks, K = a.num_topk;
+    int* s_ecnt = smem;                 // [E]
+    int* s_rcnt = s_ecnt + E;           // [R]
+    short* s_key = (short*)(s_rcnt + R);
+    short* s_rk = s_key + EP_TOKENS_PER_BLOCK * K;
+    for (int i = threadIdx.x; i < E + R; i += blockDim.x) smem[i] = 0;
+    layout_load_keys(a, s_key, s_rk);
+    __syncthreads();
+    const int n = EP_TOKENS_PER_BLOCK * K;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const int e = s_key[i];
+        if (e >= 0) atomicAdd(&s_ecnt[e], 1);
+        const int mr = master_rank(s_rk, i, K);
+        if (mr >= 0) atomicAdd(&s_rcnt[mr], 1);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < E; i += blockDim.x) a.blk_expert_cnt[(int64_t)blockIdx.x * E + i] = s_ecnt[i];
+    for (int i = threadIdx.x; i < R; i += blockDim.x) a.blk_rank_cnt[(int64_t)blockIdx.x * R + i] = s_rcnt[i];
+}
+
+// ------------------------------------------------------------------------------------------------
+// Layout pass B: exclusive prefix over blocks of every histogram column, plus column totals.
+// One workgroup owns 64 columns; its 16 waves split the rows.
+// ------------------------------------------------------------------------------------------------
+extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpLayoutArgs a) {
+    __shared__ int s_part[EP_SCAN_THREADS / WAVE][WAVE];
+    const int E = a.num_experts, R = a.num_ranks, B = a.num_blocks;
+    const int lane = lane_id(), w = wave_id();
+    const int nw = EP_SCAN_THREADS / WAVE;
+    const int col = blockIdx.x * WAVE + lane;
+    const bool live = col < E + R;
+    int* base = nullptr;
+    int stride = 0;
+    if (live) {
+        if (col < E) { base = a.blk_expert_cnt + col; stride = E; }
+        else { base = a.blk_rank_cnt + (col - E); stride = R; }
+    }
+    const int rpw = (B + nw - 1) / nw;
+    const int r0 = w * rpw, r1 = min(B, r0 + rpw);
+    int sum = 0;
+    if (live)
+        for (int r = r0; r < r1; ++r) sum += base[(int64_t)r * stride];
+    s_part[w][lane] = sum;
+    __syncthreads();
+    int off = 0, total = 0;
+    for (int i = 0; i < nw; ++i) {
+        const int v = s_part[i][lane];
+        if (i < w) off += v;
+        total += v;
+    }
+    if (live) {
+        int run = off;
+        for (int r = r0; r < r1; ++r) {
+            const int v = base[(int64_t)r * stride];
+            base[(int64_t)r * stride] = run;
+            run += v;
+        }
+        if (w == 0) {
+            if (col < E) a.expert_total[col] = total;
+            else a.rank_total[col - E] = total;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Layout pass C: slot of every entry.
+//   dst_buffer_slot_idx[t,j] = number of earlier tokens with a master for the same partition
+//                               (masters only)                       -- impls/ep/dispatch.hpp:258-281
+//   slot_map[t,j]            = expert_start[e] + number of earlier (t',j') entries with the same
+//                               local expert (lexicographic order)    -- dispatch_copy_epilogue.hpp:471-488
+//                               with the canonical order of deep_ep/buffers/ep.py:100-160
+// Block 0 also publishes the per-partition / per-expert counts and prefix sums
+// (impls/ep/dispatch.hpp:469-545) and, when asked, the host count page.
+// ------------------------------------------------------------------------------------------------
+extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign(EpLayoutArgs a) {
+    extern __shared__ int smem[];
+    const int E = a.num_experts, R = a.num_ranks, K = a.num_topk, El = a.experts_per_rank, A = a.expert_alignment;
+    const int NW = EP_LAYOUT_THREADS / WAVE;
+    int* s_start = smem;                   // [El] first slot of each local expert
+    int* s_we = s_start + El;              // [NW][E] running slot counters per wave
+    int* s_wr = s_we + NW * E;             // [NW][R]
+    int* s_tmp = s_wr + NW * R;            // [NW + 1]
+    short* s_key = (short*)(s_tmp + NW + 1);
+    short* s_rk = s_key + EP_TOKENS_PER_BLOCK * K;
+    const int tid = threadIdx.x, lane = lane_id(), w = wave_id();
+    const int lo = a.rank_idx * El;
+
+    // ---- aligned exclusive scan over the local experts (every block recomputes it: El <= 2048) ----
+    const int per = (El + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS;
+    const int e0 = tid * per, e1 = min(El, e0 + per);
+    int mine = 0;
+    for (int e = e0; e < e1; ++e) mine += align_up(a.expert_total[lo + e], A);
+    const int incl = wave_inclusive_sum(mine);
+    if (lane == WAVE - 1) s_tmp[w] = incl;
+    for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
+    layout_load_keys(a, s_key, s_rk);
+    __syncthreads();
+    int wave_off = 0, grand = 0;
+    for (int i = 0; i < NW; ++i) {
+        if (i < w) wave_off += s_tmp[i];
+        grand += s_tmp[i];
+    }
+    {
+        int run = wave_off + incl - mine;
+        for (int e = e0; e < e1; ++e) {
+            s_start[e] = run;
+            run += align_up(a.expert_total[lo + e], A);
+        }
+    }
+    __syncthreads();
+
+    if (blockIdx.x == 0) {
+        const int n_self = a.rank_total[a.rank_idx];
+        for (int e = tid; e < El; e += blockDim.x) {
+            const int c = a.expert_total[lo + e];
+            a.unaligned_expert[e] = c;
+            a.psum_expert[e] = s_start[e] + c;
+            if (a.cumulative_stats != nullptr) atomicAdd(&a.cumulative_stats[e], c);
+            if (a.notify_host) a.host_page[EP_HOST_EXPERT_OFF + e] = align_up(c, A);
+        }
+        for (int r = tid; r < R; r += blockDim.x) {
+            a.psum_rank[r] = r >= a.rank_idx ? n_self : 0;
+            if (a.notify_host) a.host_page[EP_HOST_RANK_OFF + r] = r == a.rank_idx ? n_self : 0;
+        }
+        if (a.notify_host) {
+            __threadfence_system();
+            __syncthreads();
+            if (tid == 0) {
+                a.host_page[1] = n_self;
+                a.host_page[2] = grand;
+                __threadfence_system();
+                __hip_atomic_store(&a.host_page[0], a.seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
+    }
+
+    // ---- per-wave counts: wave w owns entries [w*epw, (w+1)*epw) of this block's chunk ----
+    const int n = EP_TOKENS_PER_BLOCK * K;
+    const int rounds = (n + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS;
+    const int epw = rounds * WAVE;
+    for (int rd = 0; rd < rounds; ++rd) {
+        const int idx = w * epw + rd * WAVE + lane;
+        if (idx < n) {
+            const int e = s_key[idx];
+            if (e >= 0) atomicAdd(&s_we[w * E + e], 1);
+            const int mr = master_rank(s_rk, idx, K);
+            if (mr >= 0) atomicAdd(&s_wr[w * R + mr], 1);
+        }
+    }
+    __syncthreads();
+    // counts -> starting slots (global base + blocks before + waves before)
+    for (int e = tid; e < E; e += blockDim.x) {
+        const int le = e - lo;
+        int run = a.blk_expert_cnt[(int64_t)blockIdx.x * E + e] + ((le >= 0 && le < El) ? s_start[le] : 0);
+        for (int i = 0; i < NW; ++i) {
+            const int c = s_we[i * E + e];
+            s_we[i * E + e] = run;
+            run += c;
+        }
+    }
+    for (int r = tid; r < R; r += blockDim.x) {
+        int run = a.blk_rank_cnt[(int64_t)blockIdx.x * R + r];
+        for (int i = 0; i < NW; ++i) {
+            const int c = s_wr[i * R + r];
+            s_wr[i * R + r] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+
+    // ---- stable ranking, 64 consecutive entries per wave per round ----
+    const int ebits = 32 - __builtin_clz(E);       // keys+1 in [0, E]
+    const int rbits = 32 - __builtin_clz(R);
+    const uint64_t lt = (1ull << lane) - 1ull;
+    const int64_t total = (int64_t)a.num_tokens * K;
+    for (int rd = 0; rd < rounds; ++rd) {
+        const int idx = w * epw + rd * WAVE + lane;
+        const bool in = idx < n;
+        const int e = in ? s_key[idx] : -1;
+        const int mr = in ? master_rank(s_rk, idx, K) : -1;
+        const uint64_t pe = match_any(e + 1, ebits);
+        const uint64_t pr = match_any(mr + 1, rbits);
+        int eslot = -1, rslot = -1;
+        if (e >= 0) {
+            eslot = s_we[w * E + e] + __popcll(pe & lt);
+            if ((pe >> lane) == 1ull) s_we[w * E + e] = eslot + 1;      // highest peer advances the counter
+        }
+        if (mr >= 0) {
+            rslot = s_wr[w * R + mr] + __popcll(pr & lt);
+            if ((pr >> lane) == 1ull) s_wr[w * R + mr] = rslot + 1;
+        }
+        const int64_t g = (int64_t)blockIdx.x * n + idx;
+        if (in && g < total) {
+            const int le = e - lo;
+            a.dst_buffer_slot_idx[g] = rslot;
+            a.dst_gsge_idx[g] = -1;                 // every copy is local: no transport descriptors
+            a.slot_map[g] = (e >= 0 && le >= 0 && le < El) ? eslot : -1;
+            if (mr == a.rank_idx && rslot < a.max_tokens) a.recv_tok[rslot] = (int)(g / K);
+        }
+        __syncthreads();
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Scatter (dispatch copy epilogue): one receive-stream row per wave.
+// Reference semantics: impls/ep/dispatch_copy_epilogue.hpp:450-545 (expand), :547-620 (zero padding).
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_lo(unsigned int u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(unsigned int u) { return __uint_as_float(u & 0xffff0000u); }
+
+// max over the 16 lanes of a DPP row, result in every lane of the row
+__device__ __forceinline__ float row16_max(float v) {
+    int x = __float_as_int(v);
+    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x128, 0xf, 0xf, false))));  // row_ror:8
+    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x124, 0xf, 0xf, false))));  // row_ror:4
+    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x122, 0xf, 0xf, false))));  // row_ror:2
+    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x121, 0xf, 0xf, false))));  // row_ror:1
+    return __int_as_float(x);
+}
+
+template <bool HW>
+__device__ __forceinline__ u32x2 quant8(const float* f, float inv) {
+    u32x2 o;
+    if (HW) {
+        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0] * inv, f[1] * inv, 0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2] * inv, f[3] * inv, w0, true);
+        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4] * inv, f[5] * inv, 0, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6] * inv, f[7] * inv, w1, true);
+        o.x = (unsigned)w0;
+        o.y = (unsigned)w1;
+    } else {
+        unsigned b[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b[i] = ep_f32_bits_to_e4m3fn(__float_as_uint(f[i] * inv));
+        o.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+        o.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+    }
+    return o;
+}
+
+struct RowCtx {
+    int t;        // local token index of the row
+    int myslot;   // lane j < K: expanded slot of (row, j) or -1
+};
+
+// Resolves the row's token and slots; writes (non-cached) the metadata row and the gate weights.
+__device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int i, RowCtx& c) {
+    const int lane = lane_id();
+    const int K = a.num_topk;
+    int myslot = -1, t;
+    if (!a.cached) {
+        t = a.recv_tok[i];
+        if (t < 0 || t >= a.num_tokens) return false;
+        if (lane < K) myslot = a.slot_map[(int64_t)t * K + lane];
+        const uint64_t vm = __ballot(myslot >= 0);
+        const int master = vm == 0 ? -1 : 63 - __builtin_clzll(vm);
+        // [slot_0 .. slot_{K-1}, src_token_global_idx, last local j]  (dispatch_copy_epilogue.hpp:514-522)
+        const int v = lane < K ? myslot : (lane == K ? a.rank_idx * a.max_tokens + t : master);
+        if (lane < K + 2) a.recv_src_metadata[(int64_t)i * (K + 2) + lane] = v;
+    } else {
+        const int v = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
+        if (lane < K) myslot = v;
+        t = readlane(v, K) - a.rank_idx * a.max_tokens;
+        if (t < 0 || t >= a.num_tokens) return false;
+    }
+    if (a.recv_topk_weights != nullptr && lane < K && myslot >= 0)
+        a.recv_topk_weights[myslot] = a.topk_weights[(int64_t)t * K + lane];
+    c.t = t;
+    c.myslot = myslot;
+    return true;
+}
+
+__device__ __forceinline__ void zero_padding_rows(const EpScatterArgs& a) {
+    const int lane = lane_id(), w = wave_id();
+    const int pb = blockIdx.x - a.num_row_blocks;
+    const int e = pb / EP_PAD_BLOCKS_PER_EXPERT, part = pb % EP_PAD_BLOCKS_PER_EXPERT;
+    if (e >= a.num_local_experts) return;
+    const int end = a.psum_expert[e];
+    const int aend = align_up(end, a.expert_alignment);
+    const int nvec = (int)(a.out_row_bytes >> 4);
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int r = end + part * EP_ROWS_PER_BLOCK + w; r < aend; r += EP_PAD_BLOCKS_PER_EXPERT * EP_ROWS_PER_BLOCK) {
+        u32x4* d = (u32x4*)((char*)a.recv_x + (int64_t)r * a.out_row_bytes);
+        for (int v = lane; v < nvec; v += WAVE) d[v] = z;
+        if (a.recv_sf != nullptr) {
+            unsigned short* s = (unsigned short*)((char*)a.recv_sf + (int64_t)r * a.out_sf_row_bytes);
+            for (int p = lane; p < (int)(a.out_sf_row_bytes >> 1); p += WAVE) s[p] = 0;
+        }
+        if (a.recv_topk_weights != nullptr && lane == 0) a.recv_topk_weights[r] = 0.0f;
+    }
+}
+
+// Verbatim rows: BF16 payload, or FP8 payload with its 2-byte scale packs.
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpScatterArgs a) {
+    if ((int)blockIdx.x >= a.num_row_blocks) {
+        zero_padding_rows(a);
+        return;
+    }
+    const int lane = lane_id();
+    const int i = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
+    const int n = min(*a.num_recv_ptr, a.num_rows_bound);
+    if (i >= n) return;
+    RowCtx c;
+    if (!scatter_row_prologue(a, i, c)) return;
+    const int K = a.num_topk;
+    const int nvec = (int)(a.x_row_bytes >> 4);
+    const u32x4* src = (const u32x4*)((const char*)a.x + (int64_t)c.t * a.x_row_bytes);
+    for (int v = lane; v < nvec; v += 2 * WAVE) {
+        const bool has1 = v + WAVE < nvec;
+        const u32x4 d0 = __builtin_nontemporal_load(src + v);
+        u32x4 d1 = d0;
+        if (has1) d1 = __builtin_nontemporal_load(src + v + WAVE);
+        for (int j = 0; j < K; ++j) {
+            const int s = readlane(c.myslot, j);
+            if (s < 0) continue;
+            u32x4* dst = (u32x4*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes);
+            __builtin_nontemporal_store(d0, dst + v);
+            if (has1) __builtin_nontemporal_store(d1, dst + v + WAVE);
+        }
+    }
+    if (a.recv_sf != nullptr) {
+        const int P = a.num_sf_packs;
+        const char* sfrow = (const char*)a.sf + (int64_t)c.t * a.sf_token_stride_bytes;
+        for (int p = lane; p < P; p += WAVE) {
+            const unsigned short val = *(const unsigned short*)(sfrow + (int64_t)p * a.sf_pack_stride_bytes);
+            for (int j = 0; j < K; ++j) {
+                const int s = readlane(c.myslot, j);
+                if (s < 0) continue;
+                ((unsigned short*)((char*)a.recv_sf + (int64_t)s * a.out_sf_row_bytes))[p] = val;
+            }
+        }
+    }
+}
+
+// Fused BF16 -> e4m3fn quantisation (deep_ep/utils/math.py:30-38) + scatter.  A lane holds 8
+// channels per step, a 128-channel group is one DPP row of 16 lanes, and the row's fp32 scales
+// are staged in LDS so each slot receives them as one contiguous burst.
+template <bool HW>
+__device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
+    __shared__ float s_sf[EP_ROWS_PER_BLOCK][128];
+    if ((int)blockIdx.x >= a.num_row_blocks) {
+        zero_padding_rows(a);
+        return;
+    }
+    const int lane = lane_id(), w = wave_id();
+    const int i = blockIdx.x * EP_ROWS_PER_BLOCK + w;
+    const int n = min(*a.num_recv_ptr, a.num_rows_bound);
+    if (i >= n) return;
+    RowCtx c;
+    if (!scatter_row_prologue(a, i, c)) return;
+    const int K = a.num_topk;
+    const int nvec = a.hidden >> 3;                      // 16-byte vectors of 8 BF16
+    const u32x4* src = (const u32x4*)((const char*)a.x + (int64_t)c.t * a.x_row_bytes);
+    for (int v0 = 0; v0 < nvec; v0 += WAVE) {
+        const int v = v0 + lane;
+        const bool live = v < nvec;
+        u32x4 d = {0u, 0u, 0u, 0u};
+        if (live) d = __builtin_nontemporal_load(src + v);
+        float f[8] = {bf16_lo(d.x), bf16_hi(d.x), bf16_lo(d.y), bf16_hi(d.y),
+                      bf16_lo(d.z), bf16_hi(d.z), bf16_lo(d.w), bf16_hi(d.w)};
+        float m = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) m = fmaxf(m, fabsf(f[q]));
+        m = row16_max(m);
+        const float amax = fmaxf(m, 1e-4f);
+        const float inv = 448.0f / amax;
+        if (live && (lane & 15) == 0) s_sf[w][v >> 4] = amax / 448.0f;
+        const u32x2 q8 = quant8<HW>(f, inv);
+        if (live) {
+            for (int j = 0; j < K; ++j) {
+                const int s = readlane(c.myslot, j);
+                if (s < 0) continue;
+                u32x2* dst = (u32x2*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes);
+                __builtin_nontemporal_store(q8, dst + v);
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int P = (a.hidden + 127) >> 7;
+    for (int p = lane; p < P; p += WAVE) {
+        const float val = s_sf[w][p];
+        for (int j = 0; j < K; ++j) {
+            const int s = readlane(c.myslot, j);
+            if (s < 0) continue;
+            ((float*)((char*)a.recv_sf + (int64_t)s * a.out_sf_row_bytes))[p] = val;
+        }
+    }
+}
+
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant(EpScatterArgs a) {
+    scatter_quant_body<true>(a);
+}
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_sw(EpScatterArgs a) {
+    scatter_quant_body<false>(a);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Combine, single partition: gather the row's expanded slots, sum in fp32 in ascending slot
+// order, round once to BF16, then add the biases the same way.
+// Reference semantics: impls/ep/combine.hpp:291-324 + combine_utils.hpp:14-93 (owner side),
+// combine_reduce_epilogue.hpp:96-154 (token side); with one partition each token has one partial.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ unsigned f32_to_bf16_bits(float f) {
+    unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+__device__ __forceinline__ void unpack8(const u32x4& d, float* f) {
+    f[0] = bf16_lo(d.x); f[1] = bf16_hi(d.x); f[2] = bf16_lo(d.y); f[3] = bf16_hi(d.y);
+    f[4] = bf16_lo(d.z); f[5] = bf16_hi(d.z); f[6] = bf16_lo(d.w); f[7] = bf16_hi(d.w);
+}
+
+__device__ __forceinline__ u32x4 pack8(const float* f) {
+    u32x4 o;
+    o.x = f32_to_bf16_bits(f[0]) | (f32_to_bf16_bits(f[1]) << 16);
+    o.y = f32_to_bf16_bits(f[2]) | (f32_to_bf16_bits(f[3]) << 16);
+    o.z = f32_to_bf16_bits(f[4]) | (f32_to_bf16_bits(f[5]) << 16);
+    o.w = f32_to_bf16_bits(f[6]) | (f32_to_bf16_bits(f[7]) << 16);
+    return o;
+}
+
+// out = BF16(f32 b0 + f32 b1 + f32 partial), left to right; a single input is copied verbatim.
+__device__ __forceinline__ u32x4 add_biases(const EpCombineArgs& a, int t, int v, bool have_partial, u32x4 partial) {
+    const int64_t rowvec = a.hidden >> 3;
+    float acc[8], g[8];
+    int nin = 0;
+    u32x4 last = {0u, 0u, 0u, 0u};
+    const void* biases[2] = {a.bias_0, a.bias_1};
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        if (biases[b] == nullptr) continue;
+        last = ((const u32x4*)biases[b])[(int64_t)t * rowvec + v];
+        unpack8(last, g);
+        if (nin == 0) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; }
+        else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
+        ++nin;
+    }
+    if (have_partial) {
+        last = partial;
+        unpack8(partial, g);
+        if (nin == 0) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; }
+        else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
+        ++nin;
+    }
+    if (nin <= 1) return last;          // zero inputs -> zeros, one input -> verbatim
+    return pack8(acc);
+}
+
+// Tokens with no valid slot are never received: their output is the bias sum (or zero).
+__device__ __forceinline__ void combine_unrouted(const EpCombineArgs& a) {
+    const int lane = lane_id();
+    const int K = a.num_topk;
+    const int tb = ((int)blockIdx.x - a.num_row_blocks) * EP_ROW_THREADS + wave_id() * WAVE;
+    const int t = tb + lane;
+    bool unrouted = false;
+    if (t < a.num_tokens) {
+        unrouted = true;
+        for (int j = 0; j < K; ++j) {
+            const int64_t e = a.topk_idx[(int64_t)t * K + j];
+            if (e >= 0 && e < a.num_experts) unrouted = false;
+        }
+    }
+    uint64_t m = __ballot(unrouted);
+    const int nvec = a.hidden >> 3;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    while (m != 0) {
+        const int l = __builtin_ctzll(m);
+        m &= m - 1;
+        const int tt = tb + l;
+        for (int v = lane; v < nvec; v += WAVE)
+            ((u32x4*)a.combined_x)[(int64_t)tt * nvec + v] = add_biases(a, tt, v, false, z);
+        if (a.combined_topk_weights != nullptr && lane < K) a.combined_topk_weights[(int64_t)tt * K + lane] = 0.0f;
+    }
+}
+
+template <int KT>
+__device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
+    if ((int)blockIdx.x >= a.num_row_blocks) {
+        combine_unrouted(a);
+        return;
+    }
+    const int lane = lane_id();
+    const int K = KT > 0 ? KT : a.num_topk;
+    const int i = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
+    const int n = min(*a.num_recv_ptr, a.num_rows_bound);
+    if (i >= n) return;
+    const int mv = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
+    const int myslot = lane < K ? mv : -1;
+    const int t = readlane(mv, K) - a.rank_idx * a.max_tokens;
+    if (t < 0 || t >= a.num_tokens) return;
+    const int nvalid = __popcll(__ballot(myslot >= 0));
+    float myw = 0.0f;
+    if (a.expanded_weights != nullptr && myslot >= 0) myw = a.expanded_weights[myslot];
+    if (a.combined_topk_weights != nullptr && lane < K) a.combined_topk_weights[(int64_t)t * K + lane] = myw;
+    const int nvec = a.hidden >> 3;
+    const int64_t rowvec = nvec;
+    const u32x4* y = (const u32x4*)a.y;
+    u32x4* out = (u32x4*)a.combined_x + (int64_t)t * rowvec;
+    const bool has_bias = a.bias_0 != nullptr || a.bias_1 != nullptr;
+    for (int v = lane; v < nvec; v += WAVE) {
+        float acc[8];
+        u32x4 res = {0u, 0u, 0u, 0u};
+        if (KT > 0) {
+            u32x4 d[KT > 0 ? KT : 1];
+#pragma unroll
+            for (int j = 0; j < KT; ++j) {
+                const int s = readlane(myslot, j);
+                if (s >= 0) d[j] = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v);
+            }
+            bool first = true;
+#pragma unroll
+            for (int j = 0; j < KT; ++j) {
+                const int s = readlane(myslot, j);
+                if (s < 0) continue;
+                float g[8];
+                unpack8(d[j], g);
+                if (a.weighted) {
+                    const float wj = __int_as_float(readlane(__float_as_int(myw), j));
+                    for (int q = 0; q < 8; ++q) g[q] = g[q] * wj;
+                }
+                if (first) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; res = d[j]; first = false; }
+                else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
+            }
+        } else {
+            bool first = true;
+            for (int j = 0; j < K; ++j) {
+                const int s = readlane(myslot, j);
+                if (s < 0) continue;
+                const u32x4 dj = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v);
+                float g[8];
+                unpack8(dj, g);
+                if (a.weighted) {
+                    const float wj = __int_as_float(readlane(__float_as_int(myw), j));
+                    for (int q = 0; q < 8; ++q) g[q] = g[q] * wj;
+                }
+                if (first) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; res = dj; first = false; }
+                else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
+            }
+        }
+        if (nvalid >= 2 || (a.weighted && nvalid == 1)) res = pack8(acc);
+        if (has_bias) res = add_biases(a, t, v, true, res);
+        __builtin_nontemporal_store(res, out + v);
+    }
+}
+
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_generic(EpCombineArgs a) { combine_body<0>(a); }
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_k2(EpCombineArgs a) { combine_body<2>(a); }
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_k4(EpCombineArgs a) { combine_body<4>(a); }
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_k6(EpCombineArgs a) { combine_body<6>(a); }
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_k8(EpCombineArgs a) { combine_body<8>(a); }
+
+// ------------------------------------------------------------------------------------------------
+// Self-test: hardware e4m3fn conversion against the integer conversion over a range of fp32 bit
+// patterns.  out[0] = number of mismatches, out[1] = first mismatching pattern (if any).
+// ------------------------------------------------------------------------------------------------
+extern "C" __global__ __launch_bounds__(256) void ep_fp8_selftest(EpFp8TestArgs a) {
+    unsigned long long bad = 0, firstbad = ~0ull;
+    for (unsigned long long k = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; k < a.count;
+         k += (unsigned long long)gridDim.x * blockDim.x) {
+        const unsigned bits = (unsigned)(a.first + k);
+        const float f = __uint_as_float(bits);
+        if (!(fabsf(f) <= a.limit)) continue;
+        const unsigned hw = (unsigned)__builtin_amdgcn_cvt_pk_fp8_f32(f, 0.0f, 0, false) & 0xffu;
+        const unsigned sw = ep_f32_bits_to_e4m3fn(bits);
+        if (hw != sw) {
+            ++bad;
+            if (firstbad == ~0ull) firstbad = bits;
+        }
+    }
+    if (bad != 0) {
+        atomicAdd(&a.out[0], bad);
+        atomicMin(&a.out[1], firstbad);
+    }
+}

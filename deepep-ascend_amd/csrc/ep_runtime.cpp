@@ -1,0 +1,716 @@
+// Host runtime behind the C ABI of include/deep_ep_hip.h: argument contracts, the pooled arena,
+// the mapped count page and the launches of the ahead-of-time built gfx950 kernels through
+// hipModuleLaunchKernel.  It stands where the reference has csrc/buffers/ep.hpp (host class),
+// csrc/kernels/ep/*.hpp (launchers) and csrc/runtime/jit.hpp (run-time compiler).
+#include <hip/hip_runtime.h>
+
+#include <dlfcn.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/deep_ep_hip.h"
+#include "ep_args.h"
+#include "ep_fp8.h"
+
+namespace {
+
+constexpr int64_t kAllocAlign = 2097152;       // reference: common/compiled.hpp:48
+constexpr int kUbAlign = 32;                   // reference: common/compiled.hpp:39
+constexpr int64_t kWorkspaceBytes = 16 * 1024 * 1024;
+
+thread_local std::string g_err;
+
+struct EpError {
+    std::string msg;
+};
+
+std::string format(const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    return buf;
+}
+
+#define EP_HOST_ASSERT(cond)                                                                        \
+    do {                                                                                            \
+        if (!(cond)) throw EpError{format("Assertion exception (%s:%d): %s", __FILE_NAME__, __LINE__, #cond)}; \
+    } while (0)
+
+#define EP_HOST_UNREACHABLE(reason) \
+    throw EpError { format("Assertion exception (%s:%d): %s", __FILE_NAME__, __LINE__, reason) }
+
+#define HIP_CHECK(cmd)                                                                              \
+    do {                                                                                            \
+        const hipError_t e_ = (cmd);                                                                \
+        if (e_ != hipSuccess)                                                                       \
+            throw EpError{format("HIP runtime exception (%s:%d): Error code: %d, detail: %s", __FILE_NAME__, \
+                                 __LINE__, (int)e_, hipGetErrorString(e_))};                        \
+    } while (0)
+
+template <class F>
+int guarded(F&& f) {
+    try {
+        f();
+        return 0;
+    } catch (const EpError& e) {
+        g_err = e.msg;
+        return 1;
+    } catch (const std::exception& e) {
+        g_err = e.what();
+        return 1;
+    }
+}
+
+int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+int64_t align_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
+
+// ---- token layout (reference: layout/ep/token.hpp:9-83) -------------------------------------
+int64_t token_bytes(int hidden_bytes, int sf_bytes, int topk, bool with_metadata) {
+    int64_t meta = (int64_t)topk * 4 + (with_metadata ? align_up((int64_t)topk * 8, kUbAlign) + 4 : 0);
+    int64_t n = hidden_bytes;
+    if (sf_bytes > 0) n += align_up(sf_bytes, kUbAlign);
+    return n + align_up(meta, kUbAlign);
+}
+
+int64_t dispatch_buffer_size(int max_tokens, int hidden, int sf_packs, int topk, int elem, int ranks) {
+    return (int64_t)ranks * max_tokens * token_bytes(hidden * elem, sf_packs * 2, topk, true);
+}
+
+int64_t combine_buffer_size(int ranks, int max_tokens, int hidden, int topk) {
+    return (int64_t)std::min(topk, ranks) * max_tokens * token_bytes(hidden * 2, 0, topk, false);
+}
+
+// ---- code object ------------------------------------------------------------------------------
+struct Kernels {
+    hipModule_t module = nullptr;
+    hipFunction_t layout_count, layout_scan, layout_assign;
+    hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw;
+    hipFunction_t combine_generic, combine_k2, combine_k4, combine_k6, combine_k8;
+    hipFunction_t fp8_selftest;
+    int device = -1;
+};
+
+std::mutex g_mutex;
+Kernels g_k;
+bool g_fp8_hw = true;
+
+std::string library_dir() {
+    Dl_info info;
+    if (dladdr((void*)&library_dir, &info) == 0 || info.dli_fname == nullptr) return ".";
+    std::string p = info.dli_fname;
+    const auto pos = p.find_last_of('/');
+    return pos == std::string::npos ? "." : p.substr(0, pos);
+}
+
+void load_kernels(const char* dir) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_k.module != nullptr) return;
+    const std::string path = (dir != nullptr ? std::string(dir) : library_dir()) + "/ep_kernels.hsaco";
+    FILE* f = fopen(path.c_str(), "rb");
+    if (f == nullptr) throw EpError{"cannot open the gfx950 code object " + path + " (build it first)"};
+    fclose(f);
+    int ndev = 0;
+    HIP_CHECK(hipGetDeviceCount(&ndev));
+    if (ndev <= 0) throw EpError{"no HIP device visible: the EP kernels only run on a gfx950 GPU"};
+    HIP_CHECK(hipGetDevice(&g_k.device));
+    hipModule_t m;
+    HIP_CHECK(hipModuleLoad(&m, path.c_str()));
+    auto get = [&](hipFunction_t& fn, const char* name) { HIP_CHECK(hipModuleGetFunction(&fn, m, name)); };
+    get(g_k.layout_count, "ep_layout_count");
+    get(g_k.layout_scan, "ep_layout_scan");
+    get(g_k.layout_assign, "ep_layout_assign");
+    get(g_k.scatter_copy, "ep_scatter_copy");
+    get(g_k.scatter_quant, "ep_scatter_quant");
+    get(g_k.scatter_quant_sw, "ep_scatter_quant_sw");
+    get(g_k.combine_generic, "ep_combine_generic");
+    get(g_k.combine_k2, "ep_combine_k2");
+    get(g_k.combine_k4, "ep_combine_k4");
+    get(g_k.combine_k6, "ep_combine_k6");
+    get(g_k.combine_k8, "ep_combine_k8");
+    get(g_k.fp8_selftest, "ep_fp8_selftest");
+    g_k.module = m;
+}
+
+template <class A>
+void launch(hipFunction_t fn, unsigned grid, unsigned block, unsigned smem, void* stream, A& args) {
+    void* params[] = {&args};
+    HIP_CHECK(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, smem, (hipStream_t)stream, params, nullptr));
+}
+
+// ---- tensor contracts -------------------------------------------------------------------------
+bool present(const ep_tensor_t& t) { return t.data != nullptr; }
+
+int elem_size(int dtype) {
+    switch (dtype) {
+        case EP_DTYPE_BF16: case EP_DTYPE_I16: return 2;
+        case EP_DTYPE_FP8_E4M3: case EP_DTYPE_U8: return 1;
+        case EP_DTYPE_I32: case EP_DTYPE_F32: return 4;
+        case EP_DTYPE_I64: return 8;
+        default: return 0;
+    }
+}
+
+bool contiguous(const ep_tensor_t& t) {
+    int64_t expect = 1;
+    for (int d = t.ndim - 1; d >= 0; --d) {
+        if (t.size[d] != 1 && t.stride[d] != expect) return false;
+        expect *= t.size[d];
+    }
+    return true;
+}
+
+}  // namespace
+
+struct ep_buffer {
+    int rank_idx = 0, num_ranks = 1;
+    int64_t num_buffer_bytes = 0, num_lb_bytes = 0;
+    int cpu_timeout_secs = 300, gpu_timeout_secs = 100;
+    char* arena = nullptr;       // workspace || buffer || lb storage
+    int* host_page = nullptr;    // pinned + mapped
+    int* host_page_dev = nullptr;
+    int seq = 0;                 // sequence number of the last non-cached dispatch
+    bool destroyed = false;
+    int device = 0;
+    // state handed from ep_dispatch_launch to ep_dispatch_epilogue_launch
+    struct {
+        bool valid = false;
+        int num_tokens = 0, num_topk = 0, num_experts = 0, alignment = 0, max_tokens = 0;
+        int* slot_map = nullptr;
+        int* recv_tok = nullptr;
+        bool notified = false;
+    } last;
+
+    char* workspace() const { return arena; }
+    char* buffer() const { return arena + kWorkspaceBytes; }
+    char* lb() const { return arena + kWorkspaceBytes + num_buffer_bytes; }
+};
+
+extern "C" {
+
+const char* ep_last_error(void) { return g_err.c_str(); }
+
+int ep_init(const char* dir) {
+    return guarded([&] { load_kernels(dir); });
+}
+
+int64_t ep_get_num_allocation_alignment(void) { return kAllocAlign; }
+int64_t ep_get_num_tma_alignment(void) { return 32; }
+int64_t ep_get_num_rdma_alignment(void) { return 32; }
+
+int ep_get_num_compute_units(void) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    return n;
+}
+
+int64_t ep_get_dispatch_buffer_size(int max_tokens, int hidden, int sf_packs, int topk, int elem, int ranks) {
+    return dispatch_buffer_size(max_tokens, hidden, sf_packs, topk, elem, ranks);
+}
+
+int64_t ep_get_combine_buffer_size(int ranks, int max_tokens, int hidden, int topk) {
+    return combine_buffer_size(ranks, max_tokens, hidden, topk);
+}
+
+int64_t ep_calculate_buffer_size(int num_ranks, int max_tokens, int hidden, int num_topk, int use_fp8) {
+    int64_t out = -1;
+    const int rc = guarded([&] {
+        EP_HOST_ASSERT(num_ranks > 0);
+        EP_HOST_ASSERT(max_tokens > 0);
+        EP_HOST_ASSERT(hidden > 0);
+        EP_HOST_ASSERT(num_topk >= 0);
+        const int topk = num_topk == 0 ? 32 : num_topk;            // room for the largest top-k
+        const int sf_packs = use_fp8 ? (int)ceil_div(hidden, 32) : 0;   // the hint never sees the SF tensor
+        const int64_t d = dispatch_buffer_size(max_tokens, hidden, sf_packs, topk, use_fp8 ? 1 : 2, num_ranks);
+        const int64_t c = combine_buffer_size(num_ranks, max_tokens, hidden, topk);
+        out = align_up(std::max(d, c), kAllocAlign);
+    });
+    return rc == 0 ? out : -1;
+}
+
+void ep_host_f32_to_e4m3fn(const float* src, uint8_t* dst, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) {
+        uint32_t b;
+        memcpy(&b, src + i, 4);
+        dst[i] = (uint8_t)ep_f32_bits_to_e4m3fn(b);
+    }
+}
+
+void ep_set_fp8_hw_convert(int enable) { g_fp8_hw = enable != 0; }
+
+int ep_fp8_selftest(uint64_t first, uint64_t count, float limit, uint64_t out[2]) {
+    return guarded([&] {
+        load_kernels(nullptr);
+        unsigned long long* dev = nullptr;
+        HIP_CHECK(hipMalloc((void**)&dev, 16));
+        const unsigned long long init[2] = {0ull, ~0ull};
+        HIP_CHECK(hipMemcpy(dev, init, 16, hipMemcpyHostToDevice));
+        EpFp8TestArgs args = {first, count, dev, limit, 0};
+        launch(g_k.fp8_selftest, 4096, 256, 0, nullptr, args);
+        HIP_CHECK(hipDeviceSynchronize());
+        unsigned long long res[2];
+        HIP_CHECK(hipMemcpy(res, dev, 16, hipMemcpyDeviceToHost));
+        HIP_CHECK(hipFree(dev));
+        out[0] = res[0];
+        out[1] = res[1];
+    });
+}
+
+// ---- buffer -----------------------------------------------------------------------------------
+int ep_buffer_create(int rank_idx, int num_ranks, int64_t num_bytes, int64_t num_lb_bytes, int cpu_timeout_secs,
+                     int gpu_timeout_secs, ep_buffer_t** out) {
+    return guarded([&] {
+        EP_HOST_ASSERT(out != nullptr);
+        EP_HOST_ASSERT(num_bytes >= 0 and num_bytes % kAllocAlign == 0);
+        EP_HOST_ASSERT(num_lb_bytes >= 0 and num_lb_bytes % kAllocAlign == 0);
+        EP_HOST_ASSERT(num_ranks > 0 and num_ranks <= EP_MAX_RANKS and rank_idx >= 0 and rank_idx < num_ranks);
+        EP_HOST_ASSERT(cpu_timeout_secs > 0 and gpu_timeout_secs > 0);
+        load_kernels(nullptr);
+        auto* b = new ep_buffer();
+        b->rank_idx = rank_idx;
+        b->num_ranks = num_ranks;
+        b->num_buffer_bytes = num_bytes;
+        b->num_lb_bytes = num_lb_bytes;
+        b->cpu_timeout_secs = cpu_timeout_secs;
+        b->gpu_timeout_secs = gpu_timeout_secs;
+        try {
+            HIP_CHECK(hipGetDevice(&b->device));
+            const int64_t total = kWorkspaceBytes + num_bytes + num_lb_bytes;
+            HIP_CHECK(hipMalloc((void**)&b->arena, (size_t)total));
+            HIP_CHECK(hipMemset(b->arena, 0, (size_t)total));
+            HIP_CHECK(hipHostMalloc((void**)&b->host_page, EP_HOST_PAGE_INTS * sizeof(int), hipHostMallocMapped));
+            memset(b->host_page, 0, EP_HOST_PAGE_INTS * sizeof(int));
+            HIP_CHECK(hipHostGetDevicePointer((void**)&b->host_page_dev, b->host_page, 0));
+            HIP_CHECK(hipDeviceSynchronize());
+        } catch (...) {
+            if (b->arena != nullptr) (void)hipFree(b->arena);
+            if (b->host_page != nullptr) (void)hipHostFree(b->host_page);
+            delete b;
+            throw;
+        }
+        *out = b;
+    });
+}
+
+int ep_buffer_destroy(ep_buffer_t* b) {
+    return guarded([&] {
+        EP_HOST_ASSERT(b != nullptr);
+        EP_HOST_ASSERT(not b->destroyed);
+        HIP_CHECK(hipDeviceSynchronize());
+        HIP_CHECK(hipFree(b->arena));
+        HIP_CHECK(hipHostFree(b->host_page));
+        b->arena = nullptr;
+        b->host_page = nullptr;
+        b->destroyed = true;
+        delete b;
+    });
+}
+
+void* ep_buffer_region(ep_buffer_t* b, int which, int64_t* num_bytes) {
+    if (b == nullptr || b->destroyed) return nullptr;
+    switch (which) {
+        case 0: if (num_bytes) *num_bytes = kWorkspaceBytes; return b->workspace();
+        case 1: if (num_bytes) *num_bytes = b->num_buffer_bytes; return b->buffer();
+        case 2: if (num_bytes) *num_bytes = b->num_lb_bytes; return b->lb();
+        default: return nullptr;
+    }
+}
+
+int ep_buffer_print_memory_usage(ep_buffer_t* b) {
+    return guarded([&] {
+        EP_HOST_ASSERT(b != nullptr and not b->destroyed);
+        const double gib = 1 << 30;
+        printf("[DeepEP memory usage] rank_idx=%d, num_ranks=%d, GPU total %.3f GiB "
+               "(workspace %.3f GiB, buffer %.3f GiB, RDMA storage %.3f GiB), CPU total %.3f GiB\n",
+               b->rank_idx, b->num_ranks, (kWorkspaceBytes + b->num_buffer_bytes + b->num_lb_bytes) / gib,
+               kWorkspaceBytes / gib, b->num_buffer_bytes / gib, b->num_lb_bytes / gib, 0.0);
+        fflush(stdout);
+    });
+}
+
+// ---- dispatch ---------------------------------------------------------------------------------
+int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
+    return guarded([&] {
+        EP_HOST_ASSERT(b != nullptr and pa != nullptr);
+        EP_HOST_ASSERT(not b->destroyed);
+        const ep_dispatch_args_t& a = *pa;
+        const bool cached_mode = a.cached_mode != 0;
+        const bool do_cpu_sync = a.do_cpu_sync != 0;
+        if (cached_mode) {
+            EP_HOST_ASSERT(not do_cpu_sync and "Cannot do CPU sync with cached mode");
+            EP_HOST_ASSERT(not present(a.cumulative_local_expert_recv_stats));
+        }
+
+        // data tensor
+        EP_HOST_ASSERT(present(a.x));
+        EP_HOST_ASSERT(a.x.ndim == 2);
+        const int num_tokens = (int)a.x.size[0];
+        const int hidden = (int)a.x.size[1];
+        const int num_ranks = b->num_ranks;
+        EP_HOST_ASSERT(a.num_experts > 0 and a.num_experts <= EP_MAX_EXPERTS);
+        EP_HOST_ASSERT(a.num_experts % num_ranks == 0);
+        const int num_experts_per_rank = a.num_experts / num_ranks;
+        EP_HOST_ASSERT(contiguous(a.x));
+        EP_HOST_ASSERT(num_tokens <= a.num_max_tokens_per_rank);
+        EP_HOST_ASSERT(a.num_max_tokens_per_rank > 0);
+        EP_HOST_ASSERT(a.expert_alignment > 0);
+
+        int num_sf_packs = 0;
+        if (present(a.sf)) {
+            EP_HOST_ASSERT(not a.fused_fp8_quant);
+            EP_HOST_ASSERT(a.x.dtype == EP_DTYPE_FP8_E4M3);
+            EP_HOST_ASSERT(a.sf.ndim == 2 and a.sf.size[0] == num_tokens);
+            EP_HOST_ASSERT(elem_size(a.sf.dtype) == 2);
+            EP_HOST_ASSERT(a.sf.stride[0] == 1 or a.sf.stride[1] == 1);
+            EP_HOST_ASSERT(a.sf.stride[0] <= INT32_MAX and a.sf.stride[1] <= INT32_MAX);
+            num_sf_packs = (int)a.sf.size[1];
+        } else {
+            EP_HOST_ASSERT(a.x.dtype == EP_DTYPE_BF16);
+        }
+        const int x_elem = elem_size(a.x.dtype);
+        EP_HOST_ASSERT((int64_t)hidden * x_elem % 16 == 0);
+        if (a.fused_fp8_quant) {
+            EP_HOST_ASSERT(hidden % 8 == 0 and hidden <= 16384);
+        }
+
+        // top-k
+        EP_HOST_ASSERT(present(a.topk_idx) and a.topk_idx.ndim == 2);
+        const int num_topk = (int)a.topk_idx.size[1];
+        EP_HOST_ASSERT(a.topk_idx.size[0] == num_tokens);
+        EP_HOST_ASSERT(a.topk_idx.dtype == EP_DTYPE_I64);
+        EP_HOST_ASSERT(contiguous(a.topk_idx));
+        EP_HOST_ASSERT(num_topk > 0 and num_topk <= EP_MAX_TOPK);
+        if (present(a.topk_weights)) {
+            EP_HOST_ASSERT(a.topk_weights.ndim == 2);
+            EP_HOST_ASSERT(a.topk_weights.size[0] == num_tokens and a.topk_weights.size[1] == num_topk);
+            EP_HOST_ASSERT(contiguous(a.topk_weights));
+            EP_HOST_ASSERT(a.topk_weights.dtype == EP_DTYPE_F32);
+        }
+        if (present(a.cumulative_local_expert_recv_stats)) {
+            const auto& s = a.cumulative_local_expert_recv_stats;
+            EP_HOST_ASSERT(s.ndim == 1 and s.size[0] == num_experts_per_rank);
+            EP_HOST_ASSERT(contiguous(s));
+            EP_HOST_ASSERT(s.dtype == EP_DTYPE_I32);
+        }
+
+        // buffer size (the packed regions of csrc/buffers/ep.hpp:196-198)
+        const int packed_elem = a.fused_fp8_quant ? 1 : x_elem;
+        const int packed_sf = a.fused_fp8_quant ? 2 * (int)ceil_div(hidden, 128) : num_sf_packs;
+        EP_HOST_ASSERT(dispatch_buffer_size(a.num_max_tokens_per_rank, hidden, packed_sf, num_topk, packed_elem,
+                                            num_ranks) <= b->num_buffer_bytes);
+
+        // handle tensors
+        const auto& psum_rank = a.psum_num_recv_tokens_per_rank;
+        const auto& psum_expert = a.psum_num_recv_tokens_per_expert;
+        const auto& unaligned = a.num_unaligned_recv_tokens_per_expert;
+        EP_HOST_ASSERT(present(psum_rank) and present(psum_expert) and present(unaligned));
+        EP_HOST_ASSERT(present(a.dst_buffer_slot_idx) and present(a.dst_gsge_idx));
+        EP_HOST_ASSERT(psum_rank.ndim == 1 and psum_rank.size[0] == num_ranks);
+        EP_HOST_ASSERT(psum_expert.ndim == 1 and psum_expert.size[0] == num_experts_per_rank);
+        EP_HOST_ASSERT(unaligned.ndim == 1 and unaligned.size[0] == num_experts_per_rank);
+        EP_HOST_ASSERT(a.dst_buffer_slot_idx.ndim == 2 and a.dst_buffer_slot_idx.size[0] == num_tokens and
+                       a.dst_buffer_slot_idx.size[1] == num_topk);
+        EP_HOST_ASSERT(a.dst_gsge_idx.ndim == 2 and a.dst_gsge_idx.size[0] == num_tokens and
+                       a.dst_gsge_idx.size[1] == num_topk);
+        EP_HOST_ASSERT(contiguous(psum_rank) and contiguous(psum_expert) and contiguous(unaligned));
+        EP_HOST_ASSERT(contiguous(a.dst_buffer_slot_idx) and contiguous(a.dst_gsge_idx));
+        EP_HOST_ASSERT(psum_rank.dtype == EP_DTYPE_I32 and psum_expert.dtype == EP_DTYPE_I32);
+        EP_HOST_ASSERT(unaligned.dtype == EP_DTYPE_I32);
+        EP_HOST_ASSERT(a.dst_buffer_slot_idx.dtype == EP_DTYPE_I32 and a.dst_gsge_idx.dtype == EP_DTYPE_I32);
+
+        if (cached_mode) {
+            // the cached handle already holds the whole layout: nothing to enqueue before the epilogue
+            b->last.valid = false;
+            return;
+        }
+
+        // scratch carved from the workspace
+        const int E = a.num_experts, R = num_ranks, K = num_topk;
+        const int num_blocks = std::max<int>(1, (int)ceil_div(num_tokens, EP_TOKENS_PER_BLOCK));
+        int* ws = (int*)b->workspace();
+        int64_t off = 0;
+        auto carve = [&](int64_t n) {
+            int* p = ws + off;
+            off += align_up(std::max<int64_t>(n, 1), 64);
+            return p;
+        };
+        EpLayoutArgs la{};
+        la.expert_total = carve(E);
+        la.rank_total = carve(R);
+        la.blk_expert_cnt = carve((int64_t)num_blocks * E);
+        la.blk_rank_cnt = carve((int64_t)num_blocks * R);
+        la.slot_map = carve((int64_t)num_tokens * K);
+        la.recv_tok = carve(a.num_max_tokens_per_rank);
+        EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= kWorkspaceBytes);
+
+        la.topk_idx = (const int64_t*)a.topk_idx.data;
+        la.num_tokens = num_tokens;
+        la.num_topk = K;
+        la.num_experts = E;
+        la.num_ranks = R;
+        la.rank_idx = b->rank_idx;
+        la.expert_alignment = a.expert_alignment;
+        la.max_tokens = a.num_max_tokens_per_rank;
+        la.experts_per_rank = num_experts_per_rank;
+        la.num_blocks = num_blocks;
+        la.seq = ++b->seq;
+        la.notify_host = do_cpu_sync ? 1 : 0;
+        la.dst_buffer_slot_idx = (int*)a.dst_buffer_slot_idx.data;
+        la.dst_gsge_idx = (int*)a.dst_gsge_idx.data;
+        la.psum_rank = (int*)psum_rank.data;
+        la.psum_expert = (int*)psum_expert.data;
+        la.unaligned_expert = (int*)unaligned.data;
+        la.cumulative_stats = (int*)a.cumulative_local_expert_recv_stats.data;
+        la.host_page = b->host_page_dev;
+
+        const unsigned key_bytes = 2u * EP_TOKENS_PER_BLOCK * K * sizeof(short);
+        const unsigned smem_count = (unsigned)(E + R) * sizeof(int) + key_bytes;
+        const unsigned nw = EP_LAYOUT_THREADS / 64;
+        const unsigned smem_assign =
+            (unsigned)(num_experts_per_rank + nw * (E + R) + nw + 1) * sizeof(int) + key_bytes;
+        EP_HOST_ASSERT(smem_assign <= 64 * 1024);
+        launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, smem_count, a.stream, la);
+        launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 64), EP_SCAN_THREADS, 0, a.stream, la);
+        launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, a.stream, la);
+
+        b->last.valid = true;
+        b->last.num_tokens = num_tokens;
+        b->last.num_topk = K;
+        b->last.num_experts = E;
+        b->last.alignment = a.expert_alignment;
+        b->last.max_tokens = a.num_max_tokens_per_rank;
+        b->last.slot_map = la.slot_map;
+        b->last.recv_tok = la.recv_tok;
+        b->last.notified = do_cpu_sync;
+    });
+}
+
+int ep_dispatch_wait_counts(ep_buffer_t* b, int* num_recv_tokens, int* num_expanded_tokens, int* per_expert) {
+    return guarded([&] {
+        EP_HOST_ASSERT(b != nullptr and not b->destroyed);
+        EP_HOST_ASSERT(b->last.valid);
+        const auto deadline = std::chrono::steady_clock::now() + std::chrono::seconds(b->cpu_timeout_secs);
+        volatile int* page = b->host_page;
+        while (__atomic_load_n(&page[0], __ATOMIC_ACQUIRE) != b->seq) {
+            if (std::chrono::steady_clock::now() >= deadline) EP_HOST_UNREACHABLE("reduction timeout");
+        }
+        if (num_recv_tokens != nullptr) *num_recv_tokens = page[1];
+        if (num_expanded_tokens != nullptr) *num_expanded_tokens = page[2];
+        if (per_expert != nullptr) {
+            const int El = b->last.num_experts / b->num_ranks;
+            for (int e = 0; e < El; ++e) per_expert[e] = page[EP_HOST_EXPERT_OFF + e];
+        }
+    });
+}
+
+int ep_dispatch_worst_case_sizes(ep_buffer_t* b, int max_tokens, int num_topk, int num_experts, int alignment,
+                                 int* num_recv_tokens, int* num_expanded_tokens) {
+    return guarded([&] {
+        EP_HOST_ASSERT(b != nullptr and not b->destroyed);
+        EP_HOST_ASSERT(num_experts % b->num_ranks == 0 and alignment > 0);
+        const int El = num_experts / b->num_ranks;
+        int64_t n = (int64_t)b->num_ranks * max_tokens * std::min(num_topk, El);
+        n += (int64_t)(alignment - 1) * El;
+        n = align_up(n, alignment);
+        EP_HOST_ASSERT(n <= INT32_MAX);
+        *num_recv_tokens = b->num_ranks * max_tokens;
+        *num_expanded_tokens = (int)n;
+    });
+}
+
+int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_t* pa) {
+    return guarded([&] {
+        EP_HOST_ASSERT(b != nullptr and pa != nullptr);
+        EP_HOST_ASSERT(not b->destroyed);
+        const ep_dispatch_epilogue_args_t& a = *pa;
+        const bool cached_mode = a.cached_mode != 0;
+        EP_HOST_ASSERT(present(a.x) and a.x.ndim == 2 and contiguous(a.x));
+        const int num_tokens = (int)a.x.size[0];
+        const int hidden = (int)a.x.size[1];
+        const int K = a.num_topk;
+        const int R = b->num_ranks;
+        EP_HOST_ASSERT(K > 0 and K <= EP_MAX_TOPK);
+        EP_HOST_ASSERT(a.num_experts % R == 0);
+        const int El = a.num_experts / R;
+        const bool fused = a.fused_fp8_quant != 0;
+        EP_HOST_ASSERT(R == 1 and "partitioned receive is launched through the packed-region path");
+
+        EP_HOST_ASSERT(present(a.recv_x) and a.recv_x.ndim == 2 and a.recv_x.size[1] == hidden);
+        EP_HOST_ASSERT(contiguous(a.recv_x));
+        EP_HOST_ASSERT(a.recv_x.dtype == (fused ? (int)EP_DTYPE_FP8_E4M3 : a.x.dtype));
+        const int64_t num_expanded = a.recv_x.size[0];
+        const bool has_sf = present(a.sf) or fused;
+        int num_sf_packs = 0;
+        if (has_sf) {
+            EP_HOST_ASSERT(present(a.recv_sf) and a.recv_sf.ndim == 2 and a.recv_sf.size[0] == num_expanded);
+            if (fused) {
+                EP_HOST_ASSERT(a.recv_sf.dtype == EP_DTYPE_F32 and a.recv_sf.size[1] == ceil_div(hidden, 128));
+            } else {
+                EP_HOST_ASSERT(elem_size(a.recv_sf.dtype) == 2 and a.recv_sf.size[1] == a.sf.size[1]);
+                num_sf_packs = (int)a.sf.size[1];
+            }
+            // the copy epilogue only writes row-major scale rows (csrc/kernels/ep/dispatch.hpp:112-113)
+            EP_HOST_ASSERT(a.recv_sf.stride[1] == 1 and a.recv_sf.stride[0] == a.recv_sf.size[1]);
+        }
+        if (present(a.topk_weights)) {
+            EP_HOST_ASSERT(present(a.recv_topk_weights) and a.recv_topk_weights.ndim == 1);
+            EP_HOST_ASSERT(a.recv_topk_weights.size[0] == num_expanded and a.recv_topk_weights.dtype == EP_DTYPE_F32);
+            EP_HOST_ASSERT(a.topk_weights.size[0] == num_tokens and a.topk_weights.size[1] == K);
+        }
+        EP_HOST_ASSERT(present(a.recv_src_metadata) and a.recv_src_metadata.ndim == 2);
+        EP_HOST_ASSERT(a.recv_src_metadata.size[1] == K + 2);
+        EP_HOST_ASSERT(contiguous(a.recv_src_metadata));
+        EP_HOST_ASSERT(a.recv_src_metadata.dtype == EP_DTYPE_I32);
+        EP_HOST_ASSERT(present(a.psum_num_recv_tokens_per_rank) and a.psum_num_recv_tokens_per_rank.size[0] == R);
+        EP_HOST_ASSERT(present(a.psum_num_recv_tokens_per_expert) and a.psum_num_recv_tokens_per_expert.size[0] == El);
+        if (not cached_mode) {
+            EP_HOST_ASSERT(b->last.valid and "the copy epilogue follows its own dispatch launch");
+            EP_HOST_ASSERT(b->last.num_tokens == num_tokens and b->last.num_topk == K);
+        }
+
+        EpScatterArgs sa{};
+        sa.x = a.x.data;
+        sa.sf = a.sf.data;
+        sa.topk_weights = (const float*)a.topk_weights.data;
+        sa.slot_map = b->last.slot_map;
+        sa.recv_tok = b->last.recv_tok;
+        sa.num_recv_ptr = (const int*)a.psum_num_recv_tokens_per_rank.data + (R - 1);
+        sa.recv_src_metadata = (int*)a.recv_src_metadata.data;
+        sa.recv_x = a.recv_x.data;
+        sa.recv_sf = has_sf ? a.recv_sf.data : nullptr;
+        sa.recv_topk_weights = present(a.topk_weights) ? (float*)a.recv_topk_weights.data : nullptr;
+        sa.psum_expert = (const int*)a.psum_num_recv_tokens_per_expert.data;
+        sa.x_row_bytes = (int64_t)hidden * elem_size(a.x.dtype);
+        sa.out_row_bytes = (int64_t)hidden * elem_size(a.recv_x.dtype);
+        if (present(a.sf)) {
+            sa.sf_token_stride_bytes = a.sf.stride[0] * 2;
+            sa.sf_pack_stride_bytes = a.sf.stride[1] * 2;
+        }
+        sa.out_sf_row_bytes = has_sf ? a.recv_sf.size[1] * elem_size(a.recv_sf.dtype) : 0;
+        sa.hidden = hidden;
+        sa.num_topk = K;
+        // never walk past the rows the metadata tensor holds
+        sa.num_rows_bound = (int)std::min<int64_t>(num_tokens, a.recv_src_metadata.size[0]);
+        sa.num_tokens = num_tokens;
+        sa.rank_idx = b->rank_idx;
+        sa.max_tokens = a.num_max_tokens_per_rank;
+        sa.cached = cached_mode ? 1 : 0;
+        sa.num_sf_packs = num_sf_packs;
+        sa.num_local_experts = El;
+        sa.expert_alignment = a.expert_alignment;
+        sa.zero_padding = a.do_zero_padding ? 1 : 0;
+        sa.num_row_blocks = (int)ceil_div(sa.num_rows_bound, EP_ROWS_PER_BLOCK);
+        EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0);
+        const unsigned pad_blocks = a.do_zero_padding ? (unsigned)El * EP_PAD_BLOCKS_PER_EXPERT : 0u;
+        const unsigned grid = (unsigned)sa.num_row_blocks + pad_blocks;
+        if (grid == 0) return;
+        hipFunction_t fn = fused ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
+        launch(fn, grid, EP_ROW_THREADS, 0, a.stream, sa);
+    });
+}
+
+// ---- combine ----------------------------------------------------------------------------------
+int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
+    return guarded([&] {
+        EP_HOST_ASSERT(b != nullptr and pa != nullptr);
+        EP_HOST_ASSERT(not b->destroyed);
+        const ep_combine_args_t& a = *pa;
+        const int R = b->num_ranks;
+        EP_HOST_ASSERT(a.num_experts > 0 and a.num_experts % R == 0);
+
+        EP_HOST_ASSERT(present(a.x) and a.x.ndim == 2);
+        const int num_tokens = (int)a.x.size[0];
+        const int hidden = (int)a.x.size[1];
+        EP_HOST_ASSERT(contiguous(a.x));
+        EP_HOST_ASSERT(a.x.dtype == EP_DTYPE_BF16);
+        EP_HOST_ASSERT(hidden % 8 == 0);
+
+        EP_HOST_ASSERT(present(a.combined_topk_idx) and a.combined_topk_idx.ndim == 2);
+        const int num_combined_tokens = (int)a.combined_topk_idx.size[0];
+        const int K = (int)a.combined_topk_idx.size[1];
+        EP_HOST_ASSERT(K > 0 and K <= EP_MAX_TOPK);
+        EP_HOST_ASSERT(num_combined_tokens <= a.num_max_tokens_per_rank);
+        EP_HOST_ASSERT(contiguous(a.combined_topk_idx));
+        EP_HOST_ASSERT(a.combined_topk_idx.dtype == EP_DTYPE_I64);
+        EP_HOST_ASSERT(present(a.src_metadata) and a.src_metadata.ndim == 2 and a.src_metadata.size[1] == K + 2);
+        EP_HOST_ASSERT(a.src_metadata.size[0] <= (int64_t)R * a.num_max_tokens_per_rank);
+        EP_HOST_ASSERT(contiguous(a.src_metadata));
+        EP_HOST_ASSERT(a.src_metadata.dtype == EP_DTYPE_I32);
+        const auto& psum_rank = a.psum_num_recv_tokens_per_rank;
+        EP_HOST_ASSERT(present(psum_rank) and psum_rank.ndim == 1);
+        EP_HOST_ASSERT(psum_rank.size[0] == R);
+        EP_HOST_ASSERT(contiguous(psum_rank));
+        EP_HOST_ASSERT(psum_rank.dtype == EP_DTYPE_I32);
+
+        if (present(a.topk_weights)) {
+            EP_HOST_ASSERT(a.topk_weights.ndim == 1 and a.topk_weights.size[0] == num_tokens);
+            EP_HOST_ASSERT(contiguous(a.topk_weights));
+            EP_HOST_ASSERT(a.topk_weights.dtype == EP_DTYPE_F32);
+        }
+        EP_HOST_ASSERT(not a.apply_weights or present(a.topk_weights));
+        const ep_tensor_t* biases[2] = {&a.bias_0, &a.bias_1};
+        for (const ep_tensor_t* bias : biases) {
+            if (present(*bias)) {
+                EP_HOST_ASSERT(bias->ndim == 2);
+                EP_HOST_ASSERT(bias->size[0] == num_combined_tokens and bias->size[1] == hidden);
+                EP_HOST_ASSERT(contiguous(*bias));
+                EP_HOST_ASSERT(bias->dtype == a.x.dtype);
+            }
+        }
+        EP_HOST_ASSERT(combine_buffer_size(R, a.num_max_tokens_per_rank, hidden, K) <= b->num_buffer_bytes);
+        EP_HOST_ASSERT(phase == 0 or phase == 1);
+        EP_HOST_ASSERT(R == 1 and "partitioned combine is launched through the packed-region path");
+        if (phase == 0) return;     // single partition: the whole reduction is one token-side launch
+
+        EP_HOST_ASSERT(present(a.combined_x) and a.combined_x.ndim == 2);
+        EP_HOST_ASSERT(a.combined_x.size[0] == num_combined_tokens and a.combined_x.size[1] == hidden);
+        EP_HOST_ASSERT(contiguous(a.combined_x) and a.combined_x.dtype == EP_DTYPE_BF16);
+        if (present(a.topk_weights)) {
+            const auto& w = a.combined_topk_weights;
+            EP_HOST_ASSERT(present(w) and w.ndim == 2 and w.size[0] == num_combined_tokens and w.size[1] == K);
+            EP_HOST_ASSERT(contiguous(w) and w.dtype == EP_DTYPE_F32);
+        }
+
+        EpCombineArgs ca{};
+        ca.y = a.x.data;
+        ca.expanded_weights = (const float*)a.topk_weights.data;
+        ca.bias_0 = a.bias_0.data;
+        ca.bias_1 = a.bias_1.data;
+        ca.recv_src_metadata = (const int*)a.src_metadata.data;
+        ca.num_recv_ptr = (const int*)psum_rank.data + (R - 1);
+        ca.topk_idx = (const int64_t*)a.combined_topk_idx.data;
+        ca.combined_x = a.combined_x.data;
+        ca.combined_topk_weights = present(a.topk_weights) ? (float*)a.combined_topk_weights.data : nullptr;
+        ca.hidden = hidden;
+        ca.num_topk = K;
+        ca.num_tokens = num_combined_tokens;
+        ca.num_rows_bound = (int)a.src_metadata.size[0];
+        ca.rank_idx = b->rank_idx;
+        ca.max_tokens = a.num_max_tokens_per_rank;
+        ca.weighted = a.apply_weights ? 1 : 0;
+        ca.num_row_blocks = (int)ceil_div(ca.num_rows_bound, EP_ROWS_PER_BLOCK);
+        ca.num_experts = a.num_experts;
+        const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(num_combined_tokens, EP_ROW_THREADS);
+        if (grid == 0) return;
+        hipFunction_t fn = g_k.combine_generic;
+        switch (K) {
+            case 2: fn = g_k.combine_k2; break;
+            case 4: fn = g_k.combine_k4; break;
+            case 6: fn = g_k.combine_k6; break;
+            case 8: fn = g_k.combine_k8; break;
+            default: break;
+        }
+        launch(fn, grid, EP_ROW_THREADS, 0, a.stream, ca);
+    });
+}
+
+}  // extern "C"

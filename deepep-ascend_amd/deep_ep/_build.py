@@ -1,0 +1,39 @@
+"""Builds the two native artefacts of the package for gfx950, in-tree:
+
+  deep_ep/lib/ep_kernels.hsaco     device code object   (hipcc --genco)
+  deep_ep/lib/libdeep_ep_hip.so    host runtime, C ABI  (hipcc -shared)
+
+hipcc cross-compiles, so this runs on a machine without a GPU.  `python -m deep_ep._build`.
+"""
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(os.path.dirname(PKG), 'csrc')
+LIB = os.path.join(PKG, 'lib')
+HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
+
+DEVICE_FLAGS = [
+    '--offload-arch=gfx950', '--genco', '-O3', '-std=c++17',
+    '-ffp-contract=off',                              # combine and quantiser round every product and sum
+    '-fhip-fp32-correctly-rounded-divide-sqrt',       # 448/amax and amax/448 are IEEE divisions
+    '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+]
+HOST_FLAGS = ['-shared', '-fPIC', '-O2', '-std=c++17', '-Wall']
+
+
+def run(cmd):
+    print(' '.join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build(verbose: bool = True) -> None:
+    os.makedirs(LIB, exist_ok=True)
+    run([HIPCC, *DEVICE_FLAGS, '-o', os.path.join(LIB, 'ep_kernels.hsaco'), os.path.join(CSRC, 'ep_kernels.hip')])
+    run([HIPCC, *HOST_FLAGS, '-o', os.path.join(LIB, 'libdeep_ep_hip.so'), os.path.join(CSRC, 'ep_runtime.cpp')])
+
+
+if __name__ == '__main__':
+    build()
+    sys.exit(0)

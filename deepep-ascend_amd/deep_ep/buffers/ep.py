@@ -1,0 +1,364 @@
+"""`EPBuffer` / `EPHandle`: the expert-parallel dispatch and combine API, call-compatible with the
+reference's deep_ep/buffers/ep.py, backed by the gfx950 kernels of libdeep_ep_hip.so.
+
+One GPU's share: a group of size R describes R partitions of this GPU's arena (a
+`deep_ep.comm.LocalGroup`, or a torch ProcessGroup of size 1); there is no transport.
+Everything runs on the caller's current stream.
+"""
+import os
+from typing import Optional, Sequence, Tuple, Union
+
+import torch
+
+from .. import _C, comm
+from .._C import EventHandle
+from ..utils.event import EventOverlap
+from ..utils.semantic import value_or
+from .allocator import BufferAllocator
+from .base import BufferBase
+
+_TensorOrPair = Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]
+
+
+class EPHandle:
+    """What `EPBuffer.dispatch` learned about the routing; replays the layout in a cached dispatch
+    and reverses it in `EPBuffer.combine`.
+
+    Attributes (shapes as in the reference, deep_ep/buffers/ep.py:27-51):
+        do_expand, num_experts, expert_alignment, num_max_tokens_per_rank, num_sms: call parameters.
+        topk_idx: `[num_tokens, num_topk]` int64, held by reference; must stay unmodified.
+        psum_num_recv_tokens_per_rank: `[num_ranks]` inclusive prefix sum of received tokens
+            (a token counts once per partition however many of its experts live there).
+        psum_num_recv_tokens_per_expert: `[num_local_experts]`; entry i = aligned total of the
+            experts before i plus the exact count of expert i.
+        num_unaligned_recv_tokens_per_expert: `[num_local_experts]` exact counts.
+        num_recv_tokens_per_expert_list: aligned counts as a Python list (host-synced dispatch only).
+        recv_src_metadata: `[num_recv_tokens, num_topk + 2]` rows `[slot_0..slot_{K-1}, source
+            token, last local top-k position]`.
+        dst_buffer_slot_idx / dst_gsge_idx: `[num_tokens, num_topk]` send-side slot per partition
+            master, and transport descriptor ids (always -1: every copy is local).
+        num_recv_tokens / num_expanded_tokens: sizes of the receive stream and of the expanded
+            output (upper bounds when the dispatch did not sync with the host).
+    """
+
+    def __init__(self, do_expand: bool, num_experts: int, expert_alignment: int, num_max_tokens_per_rank: int,
+                 num_sms: int, topk_idx: torch.Tensor, num_recv_tokens: int, num_expanded_tokens: int,
+                 num_recv_tokens_per_expert_list: list, psum_num_recv_tokens_per_rank: torch.Tensor,
+                 psum_num_recv_tokens_per_expert: torch.Tensor, num_unaligned_recv_tokens_per_expert: torch.Tensor,
+                 recv_src_metadata: torch.Tensor, dst_buffer_slot_idx: torch.Tensor, dst_gsge_idx: torch.Tensor):
+        assert topk_idx is not None
+        self.do_expand = do_expand
+        self.num_experts = num_experts
+        self.expert_alignment = expert_alignment
+        self.num_max_tokens_per_rank = num_max_tokens_per_rank
+        self.num_sms = num_sms
+        self.num_recv_tokens = num_recv_tokens
+        self.num_expanded_tokens = num_expanded_tokens
+        self.num_recv_tokens_per_expert_list = num_recv_tokens_per_expert_list
+        self.psum_num_recv_tokens_per_rank = psum_num_recv_tokens_per_rank
+        self.psum_num_recv_tokens_per_expert = psum_num_recv_tokens_per_expert
+        self.num_unaligned_recv_tokens_per_expert = num_unaligned_recv_tokens_per_expert
+        self.recv_src_metadata = recv_src_metadata
+        self.dst_buffer_slot_idx = dst_buffer_slot_idx
+        self.dst_gsge_idx = dst_gsge_idx
+        self.cached_recv_src_metadata_before_sort = None
+        self._topk_idx = topk_idx
+        # inference tensors carry no version counter
+        self._topk_idx_version = None if topk_idx.is_inference() else topk_idx._version
+
+    @property
+    def topk_idx(self) -> torch.Tensor:
+        if self._topk_idx_version is not None:
+            assert self._topk_idx._version == self._topk_idx_version, \
+                '`topk_idx` must not be modified while the EP handle is in use'
+        return self._topk_idx
+
+    def deterministic_sort(self, do_cpu_sync: bool, is_cached_dispatch: bool, recv_x: torch.Tensor,
+                           recv_sf: Optional[torch.Tensor], recv_topk_weights: Optional[torch.Tensor]) -> None:
+        """The reference sorts each expert's rows by source token after the fact
+        (deep_ep/buffers/ep.py:100-160).  The layout kernels here already assign slots in that
+        order -- by (source token, top-k position) inside every expert, padding last -- so the
+        expanded tensors and `recv_src_metadata` are canonical as produced and nothing moves."""
+        if not is_cached_dispatch:
+            self.cached_recv_src_metadata_before_sort = self.recv_src_metadata
+        assert self.cached_recv_src_metadata_before_sort is not None
+
+
+class EPBuffer(BufferBase):
+    """Expert-parallel dispatch/combine with the expanded (one row per token-expert pair) layout.
+
+    Stream usage: every operation is enqueued on the current stream.
+    """
+
+    barrier = comm.barrier
+    get_comm_stream = comm.get_comm_stream
+    get_physical_domain_size = comm.get_physical_domain_size
+    get_logical_domain_size = comm.get_logical_domain_size
+
+    def __init__(self,
+                 group,
+                 num_bytes: Optional[int] = None,
+                 num_max_tokens_per_rank: int = 0,
+                 hidden: int = 0,
+                 num_topk: int = 0,
+                 use_fp8_dispatch: bool = False,
+                 lb_allocation_plan_or_num_bytes: Union[BufferAllocator, int] = 0,
+                 deterministic: bool = False,
+                 allow_hybrid_mode: bool = True,
+                 allow_multiple_reduction: bool = True,
+                 prefer_overlap_with_compute: bool = True,
+                 sl_idx: Optional[int] = None,
+                 num_allocated_qps: int = 0,
+                 num_cpu_timeout_secs: int = 300, num_gpu_timeout_secs: int = 100,
+                 explicitly_destroy: bool = False,
+                 *, use_huge1g_page: bool = True):
+        """`group` needs `rank()` and `size()`.  `num_bytes` (without workspace) must be a multiple
+        of `get_num_allocation_alignment()`; when None it comes from `get_buffer_size_hint`.
+        Load-balancing storage can be reserved; the load-balancing kernels, RDMA service levels
+        and explicit QP counts do not exist here."""
+        plan = lb_allocation_plan_or_num_bytes if isinstance(lb_allocation_plan_or_num_bytes, BufferAllocator) else None
+        num_lb_bytes = plan.num_bytes if plan is not None else lb_allocation_plan_or_num_bytes
+        if plan is not None:
+            assert not plan.materialized
+        assert isinstance(num_lb_bytes, int) and num_lb_bytes >= 0
+        assert num_lb_bytes % _C.get_num_allocation_alignment() == 0
+        if sl_idx is not None or num_allocated_qps != 0:
+            raise NotImplementedError('RDMA service levels and QP configuration are not implemented')
+        assert allow_multiple_reduction, 'allow_multiple_reduction=True is required'
+        assert num_cpu_timeout_secs > 0 and num_gpu_timeout_secs > 0
+
+        self.group = group
+        self.rank_idx, self.num_ranks = group.rank(), group.size()
+        self.allow_hybrid_mode = allow_hybrid_mode
+        self.allow_multiple_reduction = allow_multiple_reduction
+        self.prefer_overlap_with_compute = prefer_overlap_with_compute
+        self.deterministic = deterministic
+        self.num_max_tokens_per_rank = num_max_tokens_per_rank
+        self.num_allocated_qps = 0
+        self.num_lb_bytes = num_lb_bytes
+        if num_bytes is None:
+            num_bytes = self.get_buffer_size_hint(group, num_max_tokens_per_rank, hidden, num_topk,
+                                                  use_fp8_dispatch, allow_hybrid_mode, allow_multiple_reduction)
+        assert num_bytes >= 0 and num_bytes % _C.get_num_allocation_alignment() == 0
+        self.num_bytes = num_bytes
+        if os.environ.get('EP_BUFFER_DEBUG', 0):
+            print(f'Initializing EP buffer with {num_bytes} bytes at rank EP {self.rank_idx}/{self.num_ranks}')
+
+        self.hccl_comm_handle = comm.get_hccl_comm_handle(group)
+        super().__init__(explicitly_destroy)
+        self.runtime = _C.EPBuffer(self.rank_idx, self.num_ranks, self.hccl_comm_handle.get(), num_bytes,
+                                   num_lb_bytes, use_huge1g_page, num_cpu_timeout_secs, num_gpu_timeout_secs,
+                                   explicitly_destroy)
+        self.context = self.runtime.context
+        if plan is not None:
+            plan.materialize(self.runtime.lb_storage)
+        self.num_scaleout_ranks, self.num_scaleup_ranks = self.get_logical_domain_size()
+        self.scaleout_rank_idx = self.rank_idx // self.num_scaleup_ranks
+        self.scaleup_rank_idx = self.rank_idx % self.num_scaleup_ranks
+        self.num_rdma_ranks, self.num_nvlink_ranks = self.get_physical_domain_size()
+        torch.cuda.synchronize()
+
+    def destroy(self) -> None:
+        super().destroy()
+        self.context = None
+        self.hccl_comm_handle = None
+
+    @staticmethod
+    def get_buffer_size_hint(group, num_max_tokens_per_rank: int, hidden: int, num_topk: int = 0,
+                             use_fp8_dispatch: bool = False, allow_hybrid_mode: bool = True,
+                             allow_multiple_reduction: bool = True) -> int:
+        """Recommended `num_bytes` (2 MiB aligned) for these settings, without building a buffer."""
+        assert allow_multiple_reduction
+        return _C.calculate_ep_buffer_size(group.size(), num_max_tokens_per_rank, hidden, num_topk, use_fp8_dispatch)
+
+    @staticmethod
+    def capture() -> EventHandle:
+        """Record an event on the current stream."""
+        return EventHandle()
+
+    def get_theoretical_num_sms(self, num_experts: int, num_topk: int, num_scaleout_topk: int = 0,
+                                rdma_gbs: float = 0, nvlink_gbs: float = 0,
+                                sm_read_gbs: float = 0, sm_write_gbs: float = 0) -> int:
+        return _C.get_num_ai_cores()
+
+    def get_theoretical_num_qps(self, num_sms: int) -> int:
+        return 0
+
+    # ------------------------------------------------------------------------------------------
+    def dispatch(self,
+                 x: _TensorOrPair,
+                 topk_idx: Optional[torch.Tensor] = None,
+                 topk_weights: Optional[torch.Tensor] = None,
+                 cumulative_local_expert_recv_stats: Optional[torch.Tensor] = None,
+                 num_experts: Optional[int] = None,
+                 num_max_tokens_per_rank: Optional[int] = None,
+                 expert_alignment: Optional[int] = None,
+                 num_sms: int = 0,
+                 num_qps: int = 0,
+                 previous_event: Optional[EventHandle] = None,
+                 async_with_compute_stream: bool = False,
+                 allocate_on_comm_stream: bool = False,
+                 handle: Optional[EPHandle] = None,
+                 do_handle_copy: bool = False,
+                 do_cpu_sync: Optional[bool] = None,
+                 do_expand: bool = False,
+                 do_zero_padding: bool = False,
+                 use_tma_aligned_col_major_sf: bool = False,
+                 defer_epilogue: bool = False,
+                 *, fused_fp8_quant: bool = False):
+        """Send every token to the experts it selected.
+
+        Arguments (as the reference, deep_ep/buffers/ep.py:340-375):
+            x: `[num_tokens, hidden]` bfloat16, or the FP8 pair (`[num_tokens, hidden]`
+                float8_e4m3fn, `[num_tokens, num_sf_packs]` 2-byte scale packs, either stride 1).
+            topk_idx: `[num_tokens, num_topk]` int64, -1 = no selection; None with a `handle`.
+            topk_weights: `[num_tokens, num_topk]` float32, optional (also with a cached handle).
+            cumulative_local_expert_recv_stats: `[num_local_experts]` int32 running counter.
+            num_experts, num_max_tokens_per_rank, expert_alignment: layout parameters (taken
+                from the handle when one is given; alignment defaults to 1).
+            num_sms: recorded in the handle; launches size themselves.  num_qps must be 0.
+            previous_event, allocate_on_comm_stream: accepted and ignored.
+            async_with_compute_stream: also return an event for the enqueued work.
+            handle: a previous `EPHandle` to replay (no layout pass, no host sync).
+            do_cpu_sync: read exact counts on the host before allocating outputs (default True
+                without a handle); otherwise outputs have worst-case sizes.
+            do_expand: must be True.  do_handle_copy must be False.
+            do_zero_padding: zero the alignment padding rows of the outputs.
+            use_tma_aligned_col_major_sf: return the FP8 scales column-major.
+            defer_epilogue: return only the `EventOverlap`; `event.current_stream_wait()` then
+                runs the copy epilogue and returns `(recv_x, None, recv_topk_weights, handle)`.
+            fused_fp8_quant (extension): `x` is bfloat16 and is quantised to e4m3fn with one fp32
+                scale per token and 128 channels on the way; returns `(recv_x_fp8, recv_sf_fp32)`
+                whose bytes equal `per_token_cast_to_fp8(x)` dispatched verbatim.
+
+        Returns `(recv_x or (recv_x, recv_sf), None, recv_topk_weights, handle, event)`, or the
+        `EventOverlap` alone when `defer_epilogue`.
+        """
+        if num_qps not in (None, 0):
+            raise NotImplementedError('Explicit QP counts are not implemented')
+        assert not do_handle_copy, '`do_handle_copy` must be False; handle copying is no longer supported'
+        x, sf = x if isinstance(x, tuple) else (x, None)
+        assert do_expand, 'only do_expand=True is supported'
+
+        cached = handle is not None
+        if cached:
+            assert topk_idx is None
+            assert handle.do_expand == do_expand
+            assert not do_cpu_sync, 'Cannot do CPU sync with cached handle'
+            topk_idx = handle.topk_idx
+            num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, handle.num_max_tokens_per_rank)
+            num_experts = value_or(num_experts, handle.num_experts)
+            expert_alignment = value_or(expert_alignment, handle.expert_alignment)
+            assert (num_experts, expert_alignment, num_max_tokens_per_rank) == \
+                   (handle.num_experts, handle.expert_alignment, handle.num_max_tokens_per_rank)
+            num_sms, do_cpu_sync = handle.num_sms, False
+            cached_fields = (handle.num_recv_tokens, handle.num_expanded_tokens,
+                             handle.num_recv_tokens_per_expert_list, handle.psum_num_recv_tokens_per_rank,
+                             handle.psum_num_recv_tokens_per_expert, handle.num_unaligned_recv_tokens_per_expert,
+                             handle.dst_buffer_slot_idx, handle.dst_gsge_idx, handle.recv_src_metadata)
+        else:
+            if num_sms == 0:
+                num_sms = self.get_theoretical_num_sms(num_experts, topk_idx.size(1))
+            cached_fields = (None,) * 9
+        num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, self.num_max_tokens_per_rank)
+        expert_alignment = value_or(expert_alignment, 1)
+        do_cpu_sync = value_or(do_cpu_sync, True)
+
+        result, event, deferred = self.runtime.dispatch(
+            x, sf, topk_idx, topk_weights, cumulative_local_expert_recv_stats, *cached_fields,
+            num_max_tokens_per_rank, num_experts, expert_alignment, num_sms, previous_event,
+            async_with_compute_stream, allocate_on_comm_stream, do_handle_copy, do_cpu_sync, do_expand,
+            do_zero_padding, use_tma_aligned_col_major_sf, defer_epilogue, fused_fp8_quant=fused_fp8_quant)
+        overlap = EventOverlap(event)
+
+        def finalize(res: tuple, sort_in_hook: bool):
+            (recv_x, recv_sf, recv_topk_weights, num_recv_tokens, num_expanded_tokens, per_expert_list,
+             psum_rank, psum_expert, unaligned, recv_src_metadata, dst_slot, dst_gsge) = res
+            nonlocal handle
+            if not cached:
+                handle = EPHandle(do_expand, num_experts, expert_alignment, num_max_tokens_per_rank, num_sms,
+                                  topk_idx, num_recv_tokens, num_expanded_tokens, per_expert_list, psum_rank,
+                                  psum_expert, unaligned, recv_src_metadata, dst_slot, dst_gsge)
+            if self.deterministic:
+                def canonicalise():
+                    handle.deterministic_sort(do_cpu_sync, cached, recv_x, recv_sf, recv_topk_weights)
+                if sort_in_hook:
+                    overlap.register_hook_after_wait(canonicalise)
+                else:
+                    canonicalise()
+            return (recv_x, recv_sf) if recv_sf is not None else recv_x, None, recv_topk_weights, handle
+
+        if deferred is not None:
+            overlap.register_hook_after_wait(lambda: finalize(deferred(), False))
+            return overlap
+        assert result is not None
+        return (*finalize(result, async_with_compute_stream), overlap)
+
+    @staticmethod
+    def _unpack_bias(bias) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+        if isinstance(bias, torch.Tensor):
+            return bias, None
+        if isinstance(bias, tuple):
+            assert len(bias) == 2
+            return bias
+        return None, None
+
+    def combine(self,
+                x: torch.Tensor,
+                handle: EPHandle,
+                topk_weights: Optional[torch.Tensor] = None,
+                bias: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]] = None,
+                num_sms: int = 0,
+                num_qps: int = 0,
+                previous_event: EventHandle = None,
+                async_with_compute_stream: bool = False,
+                allocate_on_comm_stream: bool = False,
+                defer_epilogue: bool = False,
+                *, apply_weights: bool = False):
+        """Reduce expert outputs back to token order.
+
+        Arguments (as the reference, deep_ep/buffers/ep.py:536-550):
+            x: `[num_expanded_tokens, hidden]` bfloat16 expert outputs in the dispatch layout.
+            handle: the `EPHandle` of the dispatch being reversed.
+            topk_weights: `[num_expanded_tokens]` float32; carried back to `[num_tokens, num_topk]`.
+            bias: None, one tensor or a pair of `[num_tokens, hidden]` bfloat16 added at the end.
+            num_sms: ignored, the handle's value is used; num_qps must be 0.
+            defer_epilogue: return only the `EventOverlap`; `event.current_stream_wait()` runs the
+                final reduce and returns `(combined_x, combined_topk_weights)`.
+            apply_weights (extension): multiply each row by its gate weight before the fp32 sum
+                (the reference leaves the gate to the expert GEMM and sums rows unweighted).
+
+        Returns `(combined_x, combined_topk_weights, event)`, or the `EventOverlap` alone.
+        """
+        if num_qps not in (None, 0):
+            raise NotImplementedError('Explicit QP counts are not implemented')
+        assert handle.recv_src_metadata is not None
+        bias_0, bias_1 = self._unpack_bias(bias)
+        result, event, deferred = self.runtime.combine(
+            x, topk_weights, bias_0, bias_1, handle.recv_src_metadata, handle.topk_idx,
+            handle.psum_num_recv_tokens_per_rank, handle.num_experts, handle.num_max_tokens_per_rank,
+            handle.num_sms, previous_event, async_with_compute_stream, allocate_on_comm_stream, defer_epilogue,
+            apply_weights=apply_weights)
+        overlap = EventOverlap(event)
+        if deferred is not None:
+            overlap.register_hook_after_wait(deferred)
+            return overlap
+        assert result is not None
+        return (*result, overlap)
+
+    # ---- load-balancing entry points: storage exists, kernels do not (csrc/buffers/ep.hpp:75-86) ----
+    def lb_get_theoretical_num_sms(self) -> int:
+        return _C.get_num_ai_cores()
+
+    def lb_prefetch_weights(self, redundant_expert_weights: Union[Sequence[torch.Tensor], torch.Tensor],
+                            expert_weights: Union[Sequence[torch.Tensor], torch.Tensor],
+                            redundancy_mapping: torch.Tensor, num_sms: int = 0,
+                            previous_event: Optional[EventHandle] = None) -> EventOverlap:
+        return EventOverlap(self.runtime.lb_prefetch_weights(
+            redundant_expert_weights, expert_weights, redundancy_mapping, num_sms, previous_event))
+
+    def lb_reduce_grads(self, redundant_expert_grads: torch.Tensor, expert_grads: torch.Tensor,
+                        redundancy_mapping: torch.Tensor, num_sms: int = 0,
+                        previous_event: Optional[EventHandle] = None) -> EventOverlap:
+        return EventOverlap(self.runtime.lb_reduce_grads(
+            redundant_expert_grads, expert_grads, redundancy_mapping, num_sms, previous_event))

@@ -1,0 +1,6 @@
+from typing import Any, Optional
+
+
+def value_or(value: Optional[Any], default: Any) -> Any:
+    """`value` unless it is None."""
+    return value if value is not None else default

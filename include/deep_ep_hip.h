@@ -1,0 +1,165 @@
+/* C ABI of libdeep_ep_hip.so -- the MI355X (gfx950) implementation of the EPBuffer
+ * dispatch/combine hot path.  Plain pointers, sizes and a hipStream_t (passed as void*); no
+ * torch types.  Each entry point names the reference interface it replaces (paths relative to
+ * the reference checkout).
+ *
+ * Conventions
+ *   - every function returning int returns 0 on success; on failure it returns non-zero and
+ *     ep_last_error() gives a thread-local message.  Contract violations read
+ *     "Assertion exception (<file>:<line>): <condition>", the text the reference's EP_HOST_ASSERT
+ *     produces (deep_ep/include/deep_ep/common/exception.hpp:14-35).
+ *   - all device pointers belong to the device that was current when the buffer was created;
+ *     all kernels are enqueued on the `stream` argument and nothing synchronises unless said.
+ *   - an ep_tensor_t with data == NULL means "absent".
+ */
+#ifndef DEEP_EP_HIP_H
+#define DEEP_EP_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ep_buffer ep_buffer_t;
+
+enum ep_dtype {
+    EP_DTYPE_NONE = 0,
+    EP_DTYPE_BF16 = 1,
+    EP_DTYPE_FP8_E4M3 = 2,
+    EP_DTYPE_I16 = 3,     /* any 2-byte element: the reference's sf_pack_t */
+    EP_DTYPE_I32 = 4,
+    EP_DTYPE_I64 = 5,
+    EP_DTYPE_F32 = 6,
+    EP_DTYPE_U8 = 7
+};
+
+typedef struct ep_tensor {
+    void* data;
+    int32_t dtype;        /* enum ep_dtype */
+    int32_t ndim;         /* 1 or 2 */
+    int64_t size[2];
+    int64_t stride[2];    /* in elements */
+} ep_tensor_t;
+
+/* ---- library ------------------------------------------------------------------------------- */
+
+/* Loads the ahead-of-time built gfx950 code object `<dir>/ep_kernels.hsaco` (dir == NULL: the
+ * directory holding this library).  Replaces init_jit (csrc/runtime/jit.hpp:74-82,110-112). */
+int ep_init(const char* dir);
+const char* ep_last_error(void);
+
+/* csrc/python_api.cpp:64-73 */
+int64_t ep_get_num_allocation_alignment(void);   /* 2 MiB */
+int64_t ep_get_num_tma_alignment(void);          /* 32 */
+int64_t ep_get_num_rdma_alignment(void);         /* 32 */
+/* Compute-unit count of the current device; stands where get_num_ai_cores does
+ * (csrc/runtime/jit.hpp:89-91). */
+int ep_get_num_compute_units(void);
+
+/* EPBuffer::calculate_buffer_size (csrc/buffers/ep.hpp:581-605).  Returns -1 on a contract
+ * violation. */
+int64_t ep_calculate_buffer_size(int num_ranks, int num_max_tokens_per_rank, int hidden, int num_topk,
+                                 int use_fp8_dispatch);
+/* EPBuffer::get_dispatch_buffer_size / get_combine_buffer_size (csrc/buffers/ep.hpp:560-579). */
+int64_t ep_get_dispatch_buffer_size(int num_max_tokens_per_rank, int hidden, int num_sf_packs, int num_topk,
+                                    int element_size, int num_ranks);
+int64_t ep_get_combine_buffer_size(int num_ranks, int num_max_tokens_per_rank, int hidden, int num_topk);
+
+/* fp32 -> e4m3fn on the host with the integer algorithm the device fallback uses. */
+void ep_host_f32_to_e4m3fn(const float* src, uint8_t* dst, int64_t n);
+/* Compares the hardware conversion with the integer one over fp32 bit patterns
+ * [first, first+count) with |x| <= limit.  out[0] = mismatches, out[1] = first mismatching
+ * pattern.  Synchronises. */
+int ep_fp8_selftest(uint64_t first, uint64_t count, float limit, uint64_t out[2]);
+/* 1: hardware v_cvt_pk_fp8_f32 (default), 0: integer conversion. */
+void ep_set_fp8_hw_convert(int enable);
+
+/* ---- buffer ---------------------------------------------------------------------------------- */
+
+/* One hipMalloc'd, zero-filled arena = workspace || buffer (num_bytes) || lb storage
+ * (num_lb_bytes), plus a pinned mapped page for the receive counts.  Replaces the EPBuffer
+ * constructor and its comm::Context / SymmetricMemory (csrc/buffers/ep.hpp:36-59,
+ * csrc/kernels/comm/api.hpp:34-64, csrc/kernels/comm/symmetric.hpp:11-29). */
+int ep_buffer_create(int rank_idx, int num_ranks, int64_t num_bytes, int64_t num_lb_bytes,
+                     int num_cpu_timeout_secs, int num_gpu_timeout_secs, ep_buffer_t** out);
+/* EPBuffer::destroy (csrc/buffers/ep.hpp:65-73). */
+int ep_buffer_destroy(ep_buffer_t* buf);
+/* which: 0 workspace, 1 buffer, 2 lb storage (csrc/buffers/ep.hpp:50-53). */
+void* ep_buffer_region(ep_buffer_t* buf, int which, int64_t* num_bytes);
+/* BufferBase::print_memory_usage (csrc/buffers/base.hpp:37-49). */
+int ep_buffer_print_memory_usage(ep_buffer_t* buf);
+
+/* ---- dispatch -------------------------------------------------------------------------------- */
+
+typedef struct ep_dispatch_args {
+    /* inputs: x [T,H] BF16, or FP8 with sf [T,P] of 2-byte packs (either stride 1);
+     * topk_idx [T,K] int64 (-1 = no selection); topk_weights [T,K] fp32 (optional);
+     * cumulative_local_expert_recv_stats [E/R] int32 (optional).  csrc/buffers/ep.hpp:134-187 */
+    ep_tensor_t x, sf, topk_idx, topk_weights, cumulative_local_expert_recv_stats;
+    /* handle tensors: written in non-cached mode, only checked in cached mode (ep.hpp:205-246) */
+    ep_tensor_t psum_num_recv_tokens_per_rank;          /* [R] int32 */
+    ep_tensor_t psum_num_recv_tokens_per_expert;        /* [E/R] int32 */
+    ep_tensor_t num_unaligned_recv_tokens_per_expert;   /* [E/R] int32 */
+    ep_tensor_t dst_buffer_slot_idx;                    /* [T,K] int32 */
+    ep_tensor_t dst_gsge_idx;                           /* [T,K] int32 */
+    int32_t num_max_tokens_per_rank, num_experts, expert_alignment;
+    int32_t cached_mode, do_cpu_sync;
+    int32_t fused_fp8_quant;    /* extension: x is BF16 and is quantised to e4m3fn on the way */
+    void* stream;
+} ep_dispatch_args_t;
+
+/* Validates like EPBuffer::dispatch (csrc/buffers/ep.hpp:113-246) and enqueues the layout
+ * kernels: replaces launch_dispatch (csrc/kernels/ep/dispatch.hpp:20-82). */
+int ep_dispatch_launch(ep_buffer_t* buf, const ep_dispatch_args_t* args);
+
+/* Host wait for the counts of the last non-cached do_cpu_sync dispatch, with the buffer's CPU
+ * timeout ("reduction timeout").  per_expert receives E/R aligned counts.  Replaces the
+ * reduction::host::wait_ready loop of csrc/buffers/ep.hpp:295-315. */
+int ep_dispatch_wait_counts(ep_buffer_t* buf, int* num_recv_tokens, int* num_expanded_tokens, int* per_expert);
+/* Worst-case sizes without a host sync (csrc/buffers/ep.hpp:288,316-320). */
+int ep_dispatch_worst_case_sizes(ep_buffer_t* buf, int num_max_tokens_per_rank, int num_topk, int num_experts,
+                                 int expert_alignment, int* num_recv_tokens, int* num_expanded_tokens);
+
+typedef struct ep_dispatch_epilogue_args {
+    ep_tensor_t x, sf, topk_weights;                    /* as given to ep_dispatch_launch */
+    ep_tensor_t psum_num_recv_tokens_per_rank, psum_num_recv_tokens_per_expert;
+    ep_tensor_t recv_x;                                 /* [N_exp,H] out, dtype of x (FP8 if fused) */
+    ep_tensor_t recv_sf;                                /* [N_exp,P] out, row-major (ep.hpp:328-336) */
+    ep_tensor_t recv_topk_weights;                      /* [N_exp] fp32 out (optional) */
+    ep_tensor_t recv_src_metadata;                      /* [N_recv,K+2] int32: out, or in when cached */
+    int32_t num_topk, num_max_tokens_per_rank, num_experts, expert_alignment;
+    int32_t cached_mode, do_zero_padding, fused_fp8_quant;
+    void* stream;
+} ep_dispatch_epilogue_args_t;
+
+/* Expands every received row into its expert-major slots and zeroes the alignment padding:
+ * replaces launch_dispatch_copy_epilogue (csrc/kernels/ep/dispatch.hpp:84-139). */
+int ep_dispatch_epilogue_launch(ep_buffer_t* buf, const ep_dispatch_epilogue_args_t* args);
+
+/* ---- combine --------------------------------------------------------------------------------- */
+
+typedef struct ep_combine_args {
+    ep_tensor_t x;                      /* [N_exp,H] BF16 */
+    ep_tensor_t topk_weights;           /* [N_exp] fp32 (optional) */
+    ep_tensor_t bias_0, bias_1;         /* [T,H] BF16 (optional) */
+    ep_tensor_t src_metadata;           /* [N_recv,K+2] int32 */
+    ep_tensor_t combined_topk_idx;      /* [T,K] int64 */
+    ep_tensor_t psum_num_recv_tokens_per_rank;   /* [R] int32 */
+    ep_tensor_t combined_x;             /* [T,H] BF16 out */
+    ep_tensor_t combined_topk_weights;  /* [T,K] fp32 out (iff topk_weights) */
+    int32_t num_experts, num_max_tokens_per_rank;
+    int32_t apply_weights;              /* extension: multiply rows by their gate weight */
+    void* stream;
+} ep_combine_args_t;
+
+/* Validates like EPBuffer::combine (csrc/buffers/ep.hpp:426-481).  Replaces launch_combine and
+ * launch_combine_reduce_epilogue (csrc/kernels/ep/combine.hpp:18-112); `phase` selects which
+ * half of the reference's two launches is enqueued: 0 = owner-side reduce, 1 = token-side
+ * reduce into combined_x.  With one partition the whole reduction runs in phase 1. */
+int ep_combine_launch(ep_buffer_t* buf, const ep_combine_args_t* args, int phase);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEEP_EP_HIP_H */

@@ -429,24 +429,25 @@ def combine_fast(y: torch.Tensor, expanded_weights: Optional[torch.Tensor], meta
     started = torch.zeros(N, dtype=torch.bool)
     for j in range(K):
         m = valid[:, j]
-        rows = y[slots[m, j]]
-        acc[m] += rows.float()
-        take = m & ~started
+        take = m & ~started                          # the accumulator starts from the first row, not from +0
+        cont = m & started
         first[take] = y[slots[take, j]]
+        acc[take] = y[slots[take, j]].float()
+        acc[cont] = acc[cont] + y[slots[cont, j]].float()
         started |= m
     partial = acc.to(torch.bfloat16)
     single = nvalid == 1
     partial[single] = first[single]
     out = torch.zeros((num_tokens, H), dtype=torch.bfloat16)
     out[src] = partial
-    if bias_0 is not None or bias_1 is not None:
+    rows: List[torch.Tensor] = [b for b in (bias_0, bias_1) if b is not None]
+    if rows:
         has = torch.zeros(num_tokens, dtype=torch.bool)
         has[src] = True
-        rows: List[torch.Tensor] = [b for b in (bias_0, bias_1) if b is not None]
         acc2 = rows[0].float()
         for b in rows[1:]:
             acc2 = acc2 + b.float()
-        res = (acc2 + out.float()).to(torch.bfloat16)
+        res = torch.where(has.unsqueeze(1), acc2 + out.float(), acc2).to(torch.bfloat16)
         if len(rows) == 1:
             res[~has] = rows[0][~has]                 # one input -> verbatim copy
         out = res

@@ -1,0 +1,131 @@
+"""CPU-only checks of the native library: it loads, exports every symbol the C header declares,
+and its host-side pieces (size calculators, the integer e4m3fn conversion) agree with the oracle
+and with torch.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ep_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, 'include', 'deep_ep_hip.h')
+LIB = os.path.join(ROOT, 'deepep-ascend_amd', 'deep_ep', 'lib', 'libdeep_ep_hip.so')
+
+
+@pytest.fixture(scope='module')
+def de():
+    if not os.path.exists(LIB):
+        import __graft_entry__
+        __graft_entry__.build()
+    import deep_ep
+    return deep_ep
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(ep_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol(de):
+    lib = ctypes.CDLL(LIB)
+    names = declared_symbols()
+    assert len(names) >= 18
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_code_object_is_built_for_gfx950(de):
+    path = os.path.join(os.path.dirname(LIB), 'ep_kernels.hsaco')
+    blob = open(path, 'rb').read()
+    assert blob[:4] == b'\x7fELF' or blob.startswith(b'__CLANG_OFFLOAD_BUNDLE__')
+    for k in (b'ep_layout_count', b'ep_layout_scan', b'ep_layout_assign', b'ep_scatter_copy', b'ep_scatter_quant',
+              b'ep_combine_k6', b'ep_combine_generic', b'gfx950'):
+        assert k in blob, k
+
+
+def test_size_calculators_match_oracle(de):
+    C = de._C
+    for (R, T, H, K, fp8) in [(1, 16384, 7168, 6, False), (1, 16384, 7168, 6, True), (32, 16384, 7168, 6, True),
+                              (8, 4096, 7168, 8, False), (2, 128, 256, 0, False), (4, 7, 2048, 3, True)]:
+        assert C.calculate_ep_buffer_size(R, T, H, K, fp8) == O.calculate_buffer_size(R, T, H, K, fp8)
+    assert C.get_dispatch_buffer_size(16384, 7168, 112, 6, 1, 32) == 32 * 16384 * 7488
+    assert C.get_combine_buffer_size(32, 16384, 7168, 6) == 6 * 16384 * 14368
+    assert C.get_combine_buffer_size(2, 100, 256, 6) == 2 * 100 * (512 + 32)
+    assert (C.get_num_allocation_alignment(), C.get_num_tma_alignment(), C.get_num_rdma_alignment()) == (2097152, 32, 32)
+    assert de.topk_idx_t == torch.int64
+    with pytest.raises(C.EPException, match=r'Assertion exception \(ep_runtime.cpp:\d+\): hidden > 0'):
+        C.calculate_ep_buffer_size(1, 1, 0, 1, False)
+
+
+def test_integer_e4m3fn_conversion_matches_torch(de):
+    C = de._C
+    # all BF16 values widened to fp32 (the quantiser's inputs) times assorted scales, plus dense sweeps
+    allbf = torch.from_numpy((np.arange(65536, dtype=np.uint32) << 16).view(np.float32).copy())
+    for scale in (1.0, 448.0 / 3.0, 448.0 / 0.0123, 2.0 ** -7, 448.0 / 1e-4, 0.37):
+        f = allbf * scale
+        f = f[torch.isfinite(f)]
+        assert torch.equal(C.host_f32_to_e4m3fn(f), f.to(torch.float8_e4m3fn).view(torch.uint8)), scale
+    g = torch.Generator().manual_seed(0)
+    bits = torch.randint(0, 2 ** 31 - 1, (4_000_000,), generator=g, dtype=torch.int64).to(torch.int32)
+    f = bits.view(torch.float32)
+    f = torch.cat([f, -f])
+    f = f[torch.isfinite(f)]
+    assert torch.equal(C.host_f32_to_e4m3fn(f), f.to(torch.float8_e4m3fn).view(torch.uint8))
+    # every fp32 value in [2^-12, 512): all rounding boundaries of the format, strided
+    lo, hi = np.float32(2.0 ** -12).view(np.uint32), np.float32(512.0).view(np.uint32)
+    dense = torch.from_numpy(np.arange(lo, hi, 37, dtype=np.uint32).view(np.float32).copy())
+    assert torch.equal(C.host_f32_to_e4m3fn(dense), dense.to(torch.float8_e4m3fn).view(torch.uint8))
+    # ties exactly half way between neighbouring codes
+    codes = torch.arange(0, 0x7F, dtype=torch.uint8).view(torch.float8_e4m3fn).float()
+    mids = (codes[:-1] + codes[1:]) / 2
+    assert torch.equal(C.host_f32_to_e4m3fn(mids), mids.to(torch.float8_e4m3fn).view(torch.uint8))
+
+
+def test_no_gpu_means_loud_failure(de):
+    if torch.cuda.is_available():
+        pytest.skip('GPU present')
+    with pytest.raises(de._C.EPException, match='needs a GPU'):
+        de.EPBuffer(de.LocalGroup(), num_max_tokens_per_rank=8, hidden=64, num_topk=2)
+
+
+def test_event_overlap_runs_hook_once(de):
+    class FakeEvent:
+        waits = 0
+
+        def current_stream_wait(self):
+            FakeEvent.waits += 1
+
+    ev = de.EventOverlap(FakeEvent())
+    calls = []
+    ev.register_hook_after_wait(lambda: calls.append(1) or 'result')
+    with pytest.raises(AssertionError):
+        ev.register_hook_after_wait(lambda: None)
+    assert ev.current_stream_wait() == 'result'
+    assert ev.wait() is None and calls == [1] and FakeEvent.waits == 2
+    with ev(release_handle=True):
+        pass
+    assert ev.event is None and FakeEvent.waits == 3
+
+
+def test_buffer_allocator_plans_aligned_meta_tensors(de):
+    plan = de.BufferAllocator()
+    a = plan.allocate((3, 5), torch.float32)
+    b = plan.allocate((7,), torch.bfloat16)
+    assert a.is_meta and b.is_meta
+    assert [off for _, off in plan.allocations] == [0, 2097152]
+    assert plan.num_bytes == 2 * 2097152
+
+
+def test_python_quantiser_matches_oracle(de):
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn((32, 384), generator=g) * 3).to(torch.bfloat16)
+    q, s = de.utils.math.per_token_cast_to_fp8(x)
+    oq, os_ = O.quantise(x)
+    assert torch.equal(q.view(torch.uint8), oq) and torch.equal(s, os_)
+    back = de.utils.math.per_token_cast_back(q, s)
+    assert (back.float() - x.float()).abs().max() <= 0.07 * x.float().abs().max()
