@@ -1,0 +1,201 @@
+"""Headline benchmark: EP dispatch (fused BF16->FP8 e4m3) + BF16 combine of one GPU's share at
+16384 tokens x hidden 7168, top-6 of 256 experts, expert alignment 128.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one dispatch followed by one combine over synthetic inputs that are already resident in
+HBM.  After W warm-up steps exactly K steps are timed between two device synchronisations; the
+JSON line printed at the end carries the whole-step throughput (`value`, algorithmic bytes of both
+phases over the wall time of a step), the roofline of the dominant kernel measured with HIP events
+on the stream the kernels run on, the same for every kernel, and the CPU oracle timed on this
+machine's host cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, 'deepep-ascend_amd'), os.path.join(ROOT, 'tests')):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import numpy as np  # noqa: E402
+import torch  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+WORKLOADS = {
+    # name: (T, H, E, K, A, fp8)
+    'c3_headline': (16384, 7168, 256, 6, 128, True),
+    'c2_bf16_top8': (4096, 7168, 256, 8, 128, False),
+    'c1_small': (128, 256, 8, 2, 1, False),
+}
+
+
+def dispatch_bytes(T, H, K, n_valid, n_recv, fp8, fused):
+    s_in = 2 if (fused or not fp8) else 1
+    s_out = 1 if fp8 else 2
+    sfb = (H // 128) * 4 if fp8 else 0
+    b = T * H * s_in + T * K * (8 + 4) + n_valid * (H * s_out + sfb + 4) + n_recv * (K + 2) * 4 + 2 * T * K * 4
+    if fp8 and not fused:
+        b += T * sfb
+    return b
+
+
+def combine_bytes(T, H, K, n_valid, n_recv, n_bias, weights):
+    b = n_valid * H * 2 + T * H * 2 * (1 + n_bias) + n_recv * (K + 2) * 4 + T * K * 8
+    if weights:
+        b += n_valid * 4 + T * K * 4
+    return b
+
+
+def make_inputs(T, H, E, K, seed=0):
+    from helpers import make_routing, make_tokens
+    x = make_tokens(T, H, seed=seed, outliers=True)
+    topk, w = make_routing(T, E, K, seed=seed)
+    return x, topk, w
+
+
+def cpu_baseline(H, E, K, A, fp8, sample_tokens):
+    """The oracle on the host cores over `sample_tokens` tokens of the same workload."""
+    from oracle import ep_oracle as O
+    torch.set_num_threads(os.cpu_count())
+    x, topk, w = make_inputs(sample_tokens, H, E, K, seed=1)
+    g = torch.Generator().manual_seed(2)
+    t0 = time.perf_counter()
+    lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, sample_tokens)
+    if fp8:
+        q, s = O.quantise(x)
+        rx, rs, rw = O.rank_share_dispatch(q.numpy(), s.numpy().view(np.uint32), w.numpy(), lay)
+    else:
+        rx, rs, rw = O.rank_share_dispatch(x.view(torch.int16).numpy(), None, w.numpy(), lay)
+    t1 = time.perf_counter()
+    y = torch.randn((lay['num_expanded_tokens'], H), generator=g).to(torch.bfloat16)
+    t2 = time.perf_counter()
+    O.combine_fast(y, torch.from_numpy(rw), lay['recv_src_metadata'], sample_tokens, K)
+    t3 = time.perf_counter()
+    n_valid = int(lay['num_unaligned_recv_tokens_per_expert'].sum())
+    n_recv = lay['num_recv_tokens']
+    nbytes = dispatch_bytes(sample_tokens, H, K, n_valid, n_recv, fp8, True) + \
+        combine_bytes(sample_tokens, H, K, n_valid, n_recv, 0, True)
+    secs = (t1 - t0) + (t3 - t2)
+    return {'value': round(nbytes / secs / 1e9, 3), 'unit': 'GB/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+            'sample': f'{sample_tokens} of the workload\'s tokens, dispatch {t1 - t0:.2f} s + combine {t3 - t2:.2f} s '
+                      f'(numpy/torch-CPU oracle, os.cpu_count()={os.cpu_count()})'}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--workload', default='c3_headline', choices=sorted(WORKLOADS))
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--cpu-sample-tokens', type=int, default=2048)
+    ap.add_argument('--no-cpu-sync', action='store_true', help='dispatch without the host count wait')
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py measures one GPU\'s share of the EP path; run it with --gpus 1 (no collectives exist here)',
+              file=sys.stderr)
+        sys.exit(2)
+
+    import deep_ep
+    T, H, E, K, A, fp8 = WORKLOADS[args.workload]
+    dev = torch.device('cuda', 0)
+    torch.cuda.set_device(dev)
+    x, topk, w = make_inputs(T, H, E, K)
+    xg, tg, wg = x.to(dev), topk.to(dev), w.to(dev)
+    buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K,
+                           use_fp8_dispatch=fp8, explicitly_destroy=True)
+    kw = dict(num_experts=E, num_max_tokens_per_rank=T, expert_alignment=A, do_expand=True, do_zero_padding=True,
+              fused_fp8_quant=fp8)
+
+    def dispatch(handle=None):
+        if handle is None:
+            return buf.dispatch(xg, topk_idx=tg, topk_weights=wg, do_cpu_sync=not args.no_cpu_sync, **kw)
+        return buf.dispatch(xg, topk_weights=wg, handle=handle, do_expand=True, do_zero_padding=True,
+                            fused_fp8_quant=fp8)
+
+    recv, _, recv_w, handle, _ = dispatch()
+    n_exp = (recv[0] if fp8 else recv).size(0)
+    y = torch.randn((n_exp, H), generator=torch.Generator(device=dev).manual_seed(1), device=dev).to(torch.bfloat16)
+    torch.cuda.synchronize()
+    n_valid = int(handle.num_unaligned_recv_tokens_per_expert.sum().item())
+    n_recv = int(handle.psum_num_recv_tokens_per_rank[-1].item())
+    n_exp_exact = int(handle.psum_num_recv_tokens_per_expert[-1].item() + A - 1) // A * A
+    b_d = dispatch_bytes(T, H, K, n_valid, n_recv, fp8, fp8)
+    b_c = combine_bytes(T, H, K, n_valid, n_recv, 0, True)
+    pad_bytes = (n_exp_exact - n_valid) * (H * (1 if fp8 else 2) + ((H // 128) * 4 if fp8 else 0) + 4)
+
+    def step():
+        r, _, rw, h, _ = dispatch()
+        buf.combine(y, h, topk_weights=rw)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # per-kernel durations with events on the launch stream (the current stream): the copy kernel alone
+    # is what a cached dispatch enqueues, the combine is a single kernel, the layout is the remainder
+    def timed(fn, n):
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for a, b in evs:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return sorted(a.elapsed_time(b) * 1e3 for a, b in evs)      # microseconds
+
+    n_k = max(5, args.steps)
+    t_scatter = timed(lambda: dispatch(handle), n_k)
+    t_combine = timed(lambda: buf.combine(y, handle, topk_weights=recv_w), n_k)
+    t_dispatch_full = timed(lambda: dispatch(), n_k)
+    avg = lambda v: sum(v) / len(v)  # noqa: E731
+    us_scatter, us_combine, us_dispatch = avg(t_scatter), avg(t_combine), avg(t_dispatch_full)
+
+    def roof(name, nbytes, us):
+        gbs = nbytes / us / 1e3
+        return {'kernel': name, 'bound': 'hbm', 'achieved': round(gbs, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                'frac': round(gbs / HBM_PEAK_GBS, 4), 'traffic': None, 'us': round(us, 2), 'bytes': nbytes}
+
+    scatter_name = 'ep_scatter_quant' if fp8 else 'ep_scatter_copy'
+    kernels = [roof(scatter_name, b_d, us_scatter), roof(f'ep_combine_k{K}', b_c, us_combine)]
+    dominant = max(kernels, key=lambda k: k['us'])
+    out = {
+        'metric': 'dispatch & combine GB/s + % of HBM peak, 16384 tok x7168, top-6/256, FP8/BF16',
+        'value': round((b_d + b_c) / ms_per_step / 1e6, 1), 'unit': 'GB/s',
+        'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'fp8_e4m3+bf16 payload, fp32 accumulate' if fp8 else 'bf16 payload, fp32 accumulate',
+        'data': 'synthetic',
+        'config': {'workload': args.workload, 'tokens': T, 'hidden': H, 'experts': E, 'topk': K,
+                   'expert_alignment': A, 'partitions': 1, 'dispatch': 'fused bf16->fp8 e4m3 + per-128 fp32 scales'
+                   if fp8 else 'bf16', 'combine': 'bf16, fp32 accumulate, weights carried back, no bias',
+                   'do_zero_padding': True, 'do_cpu_sync': not args.no_cpu_sync,
+                   'num_valid_rows': n_valid, 'num_expanded_rows': n_exp_exact},
+        'roofline': {k: dominant[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'traffic')} |
+                    {'kernel': dominant['kernel']},
+        'kernels': kernels,
+        'phases': {
+            'dispatch_us': round(us_dispatch, 2), 'dispatch_layout_and_host_sync_us': round(us_dispatch - us_scatter, 2),
+            'dispatch_gbs': round(b_d / us_dispatch / 1e3, 1), 'dispatch_frac_hbm': round(b_d / us_dispatch / 1e3 / HBM_PEAK_GBS, 4),
+            'combine_us': round(us_combine, 2), 'combine_gbs': round(b_c / us_combine / 1e3, 1),
+            'combine_frac_hbm': round(b_c / us_combine / 1e3 / HBM_PEAK_GBS, 4),
+            'dispatch_bytes': b_d, 'combine_bytes': b_c, 'zero_padding_bytes_not_counted': pad_bytes,
+            'scatter_gbs_incl_padding': round((b_d + pad_bytes) / us_scatter / 1e3, 1),
+        },
+    }
+    if not args.no_cpu_baseline:
+        out['cpu_baseline'] = cpu_baseline(H, E, K, A, fp8, min(args.cpu_sample_tokens, T))
+    buf.destroy()
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

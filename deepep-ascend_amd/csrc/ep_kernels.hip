@@ -443,7 +443,7 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
         for (int q = 0; q < 8; ++q) m = fmaxf(m, fabsf(f[q]));
         m = row16_max(m);
         const float amax = fmaxf(m, 1e-4f);
-        const float inv = 448.0f / amax;
+        const float inv = (1.0f / amax) * 448.0f;       // torch evaluates `448.0 / t` as t.reciprocal() * 448.0
         if (live && (lane & 15) == 0) s_sf[w][v >> 4] = amax / 448.0f;
         const u32x2 q8 = quant8<HW>(f, inv);
         if (live) {

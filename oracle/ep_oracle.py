@@ -134,8 +134,11 @@ def quantise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """BF16 [T,H] -> (e4m3fn payload as uint8 [T,H], fp32 scales [T, ceil(H/128)]).
 
     Per (row, 128-channel group): amax over |x| in fp32 clamped below at 1e-4; payload
-    = RNE_e4m3fn( f32(x) * (448 / amax) ) with an fp32 IEEE division and an fp32
-    multiply; scale = amax / 448 (fp32 IEEE division).  math.py:33-38.
+    = RNE_e4m3fn( f32(x) * inv ), scale = amax / 448 (fp32 IEEE division).  math.py:33-38.
+    `inv` is what torch makes of the reference's `448.0 / amax_tensor`: Tensor.__rtruediv__
+    evaluates it as amax.reciprocal() * 448.0, i.e. fl(fl(1/amax) * 448) with two fp32
+    roundings, which differs from a single division in the last bit for some amax (the golden
+    vectors from the reference's math.py pin this).
     """
     assert x.dim() == 2 and x.dtype == torch.bfloat16
     m, n = x.shape

@@ -119,7 +119,17 @@ def test_quantise_closed_forms():
     assert s[1, 0].item() == 4.0
     assert q[1, :5].tolist() == [0x7E, 0xFE, 0x3C, 0x08, 0x01]
     assert s[1, 1].item() == np.float32(np.float32(1e-4) / np.float32(448.0))
-    # multiply-by-reciprocal, not divide-by-scale: find a value where the two differ and check which one we took
+    # the multiplier is fl(fl(1/amax) * 448), two roundings (torch's `448.0 / tensor`), not one division
+    am = np.float32(1.046875)
+    two_step = np.float32(np.float32(1) / am) * np.float32(448)
+    assert two_step != np.float32(448) / am
+    xs = torch.zeros((1, 128), dtype=torch.bfloat16)
+    xs[0, 0] = float(am)
+    xs[0, 1:] = torch.linspace(0.01, 1.04, 127).to(torch.bfloat16)
+    qs, _ = O.quantise(xs)
+    want = torch.from_numpy((xs.float().numpy() * two_step).astype(np.float32)).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert torch.equal(qs, want)
+    # multiply-by-reciprocal, not divide-by-scale
     g = torch.Generator().manual_seed(5)
     xx = (torch.randn((64, 128), generator=g) * 7).to(torch.bfloat16)
     q, s = O.quantise(xx)
