@@ -74,6 +74,8 @@ struct EpScatterArgs {
     int zero_padding;
     int num_row_blocks;           // blocks [0, num_row_blocks) copy rows, the rest zero padding
     int num_tokens;               // T: bound of the token indices a row may name
+    int num_parts;                // column parts per row; a wave task is (row, part)
+    int pad0;
 };
 
 // Fused single-partition combine: one receive-stream row per wave.
@@ -91,7 +93,8 @@ struct EpCombineArgs {
     int rank_idx, max_tokens;
     int weighted;                 // opt-in: multiply by the gate weight before summing
     int num_row_blocks;           // blocks [0, num_row_blocks) reduce rows, the rest handle unrouted tokens
-    int num_experts, pad0;
+    int num_experts;
+    int num_parts;                // 1024-channel parts per row; a wave task is (row, part)
 };
 
 // Hardware vs integer e4m3fn conversion over fp32 bit patterns [first, first+count).

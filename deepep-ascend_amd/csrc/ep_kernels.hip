@@ -323,8 +323,9 @@ struct RowCtx {
     int myslot;   // lane j < K: expanded slot of (row, j) or -1
 };
 
-// Resolves the row's token and slots; writes (non-cached) the metadata row and the gate weights.
-__device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int i, RowCtx& c) {
+// A wave task is (receive-stream row, column part).  Resolves the row's token and slots; the task
+// of part 0 also writes (non-cached) the metadata row and scatters the gate weights.
+__device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int i, int part, RowCtx& c) {
     const int lane = lane_id();
     const int K = a.num_topk;
     int myslot = -1, t;
@@ -332,18 +333,20 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
         t = a.recv_tok[i];
         if (t < 0 || t >= a.num_tokens) return false;
         if (lane < K) myslot = a.slot_map[(int64_t)t * K + lane];
-        const uint64_t vm = __ballot(myslot >= 0);
-        const int master = vm == 0 ? -1 : 63 - __builtin_clzll(vm);
-        // [slot_0 .. slot_{K-1}, src_token_global_idx, last local j]  (dispatch_copy_epilogue.hpp:514-522)
-        const int v = lane < K ? myslot : (lane == K ? a.rank_idx * a.max_tokens + t : master);
-        if (lane < K + 2) a.recv_src_metadata[(int64_t)i * (K + 2) + lane] = v;
+        if (part == 0) {
+            const uint64_t vm = __ballot(myslot >= 0);
+            const int master = vm == 0 ? -1 : 63 - __builtin_clzll(vm);
+            // [slot_0 .. slot_{K-1}, src_token_global_idx, last local j]  (dispatch_copy_epilogue.hpp:514-522)
+            const int v = lane < K ? myslot : (lane == K ? a.rank_idx * a.max_tokens + t : master);
+            if (lane < K + 2) a.recv_src_metadata[(int64_t)i * (K + 2) + lane] = v;
+        }
     } else {
         const int v = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
         if (lane < K) myslot = v;
         t = readlane(v, K) - a.rank_idx * a.max_tokens;
         if (t < 0 || t >= a.num_tokens) return false;
     }
-    if (a.recv_topk_weights != nullptr && lane < K && myslot >= 0)
+    if (part == 0 && a.recv_topk_weights != nullptr && lane < K && myslot >= 0)
         a.recv_topk_weights[myslot] = a.topk_weights[(int64_t)t * K + lane];
     c.t = t;
     c.myslot = myslot;
@@ -361,7 +364,7 @@ __device__ __forceinline__ void zero_padding_rows(const EpScatterArgs& a) {
     const u32x4 z = {0u, 0u, 0u, 0u};
     for (int r = end + part * EP_ROWS_PER_BLOCK + w; r < aend; r += EP_PAD_BLOCKS_PER_EXPERT * EP_ROWS_PER_BLOCK) {
         u32x4* d = (u32x4*)((char*)a.recv_x + (int64_t)r * a.out_row_bytes);
-        for (int v = lane; v < nvec; v += WAVE) d[v] = z;
+        for (int v = lane; v < nvec; v += WAVE) __builtin_nontemporal_store(z, d + v);
         if (a.recv_sf != nullptr) {
             unsigned short* s = (unsigned short*)((char*)a.recv_sf + (int64_t)r * a.out_sf_row_bytes);
             for (int p = lane; p < (int)(a.out_sf_row_bytes >> 1); p += WAVE) s[p] = 0;
@@ -370,35 +373,33 @@ __device__ __forceinline__ void zero_padding_rows(const EpScatterArgs& a) {
     }
 }
 
-// Verbatim rows: BF16 payload, or FP8 payload with its 2-byte scale packs.
+// Verbatim rows: BF16 payload, or FP8 payload with its 2-byte scale packs.  A task moves 1 KiB of
+// the row (16 bytes per lane) to every slot; many short tasks keep far more loads in flight than
+// one wave walking a whole row.
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpScatterArgs a) {
     if ((int)blockIdx.x >= a.num_row_blocks) {
         zero_padding_rows(a);
         return;
     }
     const int lane = lane_id();
-    const int i = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
+    const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
+    const int i = task / a.num_parts, part = task - i * a.num_parts;
     const int n = min(*a.num_recv_ptr, a.num_rows_bound);
     if (i >= n) return;
     RowCtx c;
-    if (!scatter_row_prologue(a, i, c)) return;
+    if (!scatter_row_prologue(a, i, part, c)) return;
     const int K = a.num_topk;
     const int nvec = (int)(a.x_row_bytes >> 4);
-    const u32x4* src = (const u32x4*)((const char*)a.x + (int64_t)c.t * a.x_row_bytes);
-    for (int v = lane; v < nvec; v += 2 * WAVE) {
-        const bool has1 = v + WAVE < nvec;
-        const u32x4 d0 = __builtin_nontemporal_load(src + v);
-        u32x4 d1 = d0;
-        if (has1) d1 = __builtin_nontemporal_load(src + v + WAVE);
+    const int v = part * WAVE + lane;
+    if (v < nvec) {
+        const u32x4 d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + (int64_t)c.t * a.x_row_bytes) + v);
         for (int j = 0; j < K; ++j) {
             const int s = readlane(c.myslot, j);
             if (s < 0) continue;
-            u32x4* dst = (u32x4*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes);
-            __builtin_nontemporal_store(d0, dst + v);
-            if (has1) __builtin_nontemporal_store(d1, dst + v + WAVE);
+            __builtin_nontemporal_store(d, (u32x4*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes) + v);
         }
     }
-    if (a.recv_sf != nullptr) {
+    if (part == 0 && a.recv_sf != nullptr) {
         const int P = a.num_sf_packs;
         const char* sfrow = (const char*)a.sf + (int64_t)c.t * a.sf_token_stride_bytes;
         for (int p = lane; p < P; p += WAVE) {
@@ -412,60 +413,45 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
     }
 }
 
-// Fused BF16 -> e4m3fn quantisation (deep_ep/utils/math.py:30-38) + scatter.  A lane holds 8
-// channels per step, a 128-channel group is one DPP row of 16 lanes, and the row's fp32 scales
-// are staged in LDS so each slot receives them as one contiguous burst.
+// Fused BF16 -> e4m3fn quantisation (deep_ep/utils/math.py:30-38) + scatter.  A task owns 512
+// channels of a row: a lane holds 8 of them, a 128-channel group is one DPP row of 16 lanes, so the
+// task produces 512 payload bytes and 4 fp32 scales per slot.
 template <bool HW>
 __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
-    __shared__ float s_sf[EP_ROWS_PER_BLOCK][128];
     if ((int)blockIdx.x >= a.num_row_blocks) {
         zero_padding_rows(a);
         return;
     }
-    const int lane = lane_id(), w = wave_id();
-    const int i = blockIdx.x * EP_ROWS_PER_BLOCK + w;
+    const int lane = lane_id();
+    const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
+    const int i = task / a.num_parts, part = task - i * a.num_parts;
     const int n = min(*a.num_recv_ptr, a.num_rows_bound);
     if (i >= n) return;
     RowCtx c;
-    if (!scatter_row_prologue(a, i, c)) return;
+    if (!scatter_row_prologue(a, i, part, c)) return;
     const int K = a.num_topk;
     const int nvec = a.hidden >> 3;                      // 16-byte vectors of 8 BF16
-    const u32x4* src = (const u32x4*)((const char*)a.x + (int64_t)c.t * a.x_row_bytes);
-    for (int v0 = 0; v0 < nvec; v0 += WAVE) {
-        const int v = v0 + lane;
-        const bool live = v < nvec;
-        u32x4 d = {0u, 0u, 0u, 0u};
-        if (live) d = __builtin_nontemporal_load(src + v);
-        float f[8] = {bf16_lo(d.x), bf16_hi(d.x), bf16_lo(d.y), bf16_hi(d.y),
-                      bf16_lo(d.z), bf16_hi(d.z), bf16_lo(d.w), bf16_hi(d.w)};
-        float m = 0.0f;
+    const int v = part * WAVE + lane;
+    const bool live = v < nvec;
+    u32x4 d = {0u, 0u, 0u, 0u};
+    if (live) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + (int64_t)c.t * a.x_row_bytes) + v);
+    float f[8] = {bf16_lo(d.x), bf16_hi(d.x), bf16_lo(d.y), bf16_hi(d.y),
+                  bf16_lo(d.z), bf16_hi(d.z), bf16_lo(d.w), bf16_hi(d.w)};
+    float m = 0.0f;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) m = fmaxf(m, fabsf(f[q]));
-        m = row16_max(m);
-        const float amax = fmaxf(m, 1e-4f);
-        const float inv = (1.0f / amax) * 448.0f;       // torch evaluates `448.0 / t` as t.reciprocal() * 448.0
-        if (live && (lane & 15) == 0) s_sf[w][v >> 4] = amax / 448.0f;
-        const u32x2 q8 = quant8<HW>(f, inv);
-        if (live) {
-            for (int j = 0; j < K; ++j) {
-                const int s = readlane(c.myslot, j);
-                if (s < 0) continue;
-                u32x2* dst = (u32x2*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes);
-                __builtin_nontemporal_store(q8, dst + v);
-            }
-        }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int P = (a.hidden + 127) >> 7;
-    for (int p = lane; p < P; p += WAVE) {
-        const float val = s_sf[w][p];
-        for (int j = 0; j < K; ++j) {
-            const int s = readlane(c.myslot, j);
-            if (s < 0) continue;
-            ((float*)((char*)a.recv_sf + (int64_t)s * a.out_sf_row_bytes))[p] = val;
-        }
+    for (int q = 0; q < 8; ++q) m = fmaxf(m, fabsf(f[q]));
+    m = row16_max(m);
+    const float amax = fmaxf(m, 1e-4f);
+    const float inv = (1.0f / amax) * 448.0f;       // torch evaluates `448.0 / t` as t.reciprocal() * 448.0
+    const float scale = amax / 448.0f;
+    const u32x2 q8 = quant8<HW>(f, inv);
+    if (!live) return;
+    const bool writes_scale = (lane & 15) == 0;
+    for (int j = 0; j < K; ++j) {
+        const int s = readlane(c.myslot, j);
+        if (s < 0) continue;
+        __builtin_nontemporal_store(q8, (u32x2*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes) + v);
+        if (writes_scale) ((float*)((char*)a.recv_sf + (int64_t)s * a.out_sf_row_bytes))[v >> 4] = scale;
     }
 }
 
@@ -557,6 +543,8 @@ __device__ __forceinline__ void combine_unrouted(const EpCombineArgs& a) {
     }
 }
 
+// A wave task is (receive-stream row, 1024-channel part): two 16-byte vectors per lane and slot,
+// all K*2 loads issued before the first add.
 template <int KT>
 __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     if ((int)blockIdx.x >= a.num_row_blocks) {
@@ -565,7 +553,8 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     }
     const int lane = lane_id();
     const int K = KT > 0 ? KT : a.num_topk;
-    const int i = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
+    const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
+    const int i = task / a.num_parts, part = task - i * a.num_parts;
     const int n = min(*a.num_recv_ptr, a.num_rows_bound);
     if (i >= n) return;
     const int mv = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
@@ -575,55 +564,81 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     const int nvalid = __popcll(__ballot(myslot >= 0));
     float myw = 0.0f;
     if (a.expanded_weights != nullptr && myslot >= 0) myw = a.expanded_weights[myslot];
-    if (a.combined_topk_weights != nullptr && lane < K) a.combined_topk_weights[(int64_t)t * K + lane] = myw;
+    if (part == 0 && a.combined_topk_weights != nullptr && lane < K)
+        a.combined_topk_weights[(int64_t)t * K + lane] = myw;
     const int nvec = a.hidden >> 3;
     const int64_t rowvec = nvec;
     const u32x4* y = (const u32x4*)a.y;
     u32x4* out = (u32x4*)a.combined_x + (int64_t)t * rowvec;
     const bool has_bias = a.bias_0 != nullptr || a.bias_1 != nullptr;
-    for (int v = lane; v < nvec; v += WAVE) {
-        float acc[8];
-        u32x4 res = {0u, 0u, 0u, 0u};
-        if (KT > 0) {
-            u32x4 d[KT > 0 ? KT : 1];
+    const int v0 = part * 2 * WAVE + lane, v1 = v0 + WAVE;
+    const bool live0 = v0 < nvec, live1 = v1 < nvec;
+    float acc0[8], acc1[8];
+    u32x4 res0 = {0u, 0u, 0u, 0u}, res1 = {0u, 0u, 0u, 0u};
+    if (KT > 0) {
+        u32x4 d0[KT > 0 ? KT : 1], d1[KT > 0 ? KT : 1];
 #pragma unroll
-            for (int j = 0; j < KT; ++j) {
-                const int s = readlane(myslot, j);
-                if (s >= 0) d[j] = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v);
-            }
-            bool first = true;
+        for (int j = 0; j < KT; ++j) {
+            const int s = readlane(myslot, j);
+            if (s < 0) continue;
+            if (live0) d0[j] = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v0);
+            if (live1) d1[j] = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v1);
+        }
+        bool first = true;
 #pragma unroll
-            for (int j = 0; j < KT; ++j) {
-                const int s = readlane(myslot, j);
-                if (s < 0) continue;
-                float g[8];
-                unpack8(d[j], g);
-                if (a.weighted) {
-                    const float wj = __int_as_float(readlane(__float_as_int(myw), j));
-                    for (int q = 0; q < 8; ++q) g[q] = g[q] * wj;
-                }
-                if (first) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; res = d[j]; first = false; }
-                else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
+        for (int j = 0; j < KT; ++j) {
+            const int s = readlane(myslot, j);
+            if (s < 0) continue;
+            float g0[8], g1[8];
+            unpack8(d0[j], g0);
+            unpack8(d1[j], g1);
+            if (a.weighted) {
+                const float wj = __int_as_float(readlane(__float_as_int(myw), j));
+                for (int q = 0; q < 8; ++q) { g0[q] = g0[q] * wj; g1[q] = g1[q] * wj; }
             }
-        } else {
-            bool first = true;
-            for (int j = 0; j < K; ++j) {
-                const int s = readlane(myslot, j);
-                if (s < 0) continue;
-                const u32x4 dj = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v);
-                float g[8];
-                unpack8(dj, g);
-                if (a.weighted) {
-                    const float wj = __int_as_float(readlane(__float_as_int(myw), j));
-                    for (int q = 0; q < 8; ++q) g[q] = g[q] * wj;
-                }
-                if (first) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; res = dj; first = false; }
-                else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
+            if (first) {
+                for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; }
+                res0 = d0[j]; res1 = d1[j];
+                first = false;
+            } else {
+                for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; }
             }
         }
-        if (nvalid >= 2 || (a.weighted && nvalid == 1)) res = pack8(acc);
-        if (has_bias) res = add_biases(a, t, v, true, res);
-        __builtin_nontemporal_store(res, out + v);
+    } else {
+        bool first = true;
+        for (int j = 0; j < K; ++j) {
+            const int s = readlane(myslot, j);
+            if (s < 0) continue;
+            u32x4 e0 = {0u, 0u, 0u, 0u}, e1 = {0u, 0u, 0u, 0u};
+            if (live0) e0 = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v0);
+            if (live1) e1 = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v1);
+            float g0[8], g1[8];
+            unpack8(e0, g0);
+            unpack8(e1, g1);
+            if (a.weighted) {
+                const float wj = __int_as_float(readlane(__float_as_int(myw), j));
+                for (int q = 0; q < 8; ++q) { g0[q] = g0[q] * wj; g1[q] = g1[q] * wj; }
+            }
+            if (first) {
+                for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; }
+                res0 = e0; res1 = e1;
+                first = false;
+            } else {
+                for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; }
+            }
+        }
+    }
+    if (nvalid >= 2 || (a.weighted && nvalid == 1)) {
+        res0 = pack8(acc0);
+        res1 = pack8(acc1);
+    }
+    if (live0) {
+        if (has_bias) res0 = add_biases(a, t, v0, true, res0);
+        __builtin_nontemporal_store(res0, out + v0);
+    }
+    if (live1) {
+        if (has_bias) res1 = add_biases(a, t, v1, true, res1);
+        __builtin_nontemporal_store(res1, out + v1);
     }
 }
 

@@ -608,7 +608,9 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.num_local_experts = El;
         sa.expert_alignment = a.expert_alignment;
         sa.zero_padding = a.do_zero_padding ? 1 : 0;
-        sa.num_row_blocks = (int)ceil_div(sa.num_rows_bound, EP_ROWS_PER_BLOCK);
+        // a wave task covers 1 KiB of a verbatim row, or 512 channels of a row being quantised
+        sa.num_parts = (int)std::max<int64_t>(1, fused ? ceil_div(hidden, 512) : ceil_div(sa.x_row_bytes, 1024));
+        sa.num_row_blocks = (int)ceil_div((int64_t)sa.num_rows_bound * sa.num_parts, EP_ROWS_PER_BLOCK);
         EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0);
         const unsigned pad_blocks = a.do_zero_padding ? (unsigned)El * EP_PAD_BLOCKS_PER_EXPERT : 0u;
         const unsigned grid = (unsigned)sa.num_row_blocks + pad_blocks;
@@ -697,7 +699,8 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
         ca.rank_idx = b->rank_idx;
         ca.max_tokens = a.num_max_tokens_per_rank;
         ca.weighted = a.apply_weights ? 1 : 0;
-        ca.num_row_blocks = (int)ceil_div(ca.num_rows_bound, EP_ROWS_PER_BLOCK);
+        ca.num_parts = (int)std::max<int64_t>(1, ceil_div(hidden, 1024));
+        ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
         ca.num_experts = a.num_experts;
         const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(num_combined_tokens, EP_ROW_THREADS);
         if (grid == 0) return;
