@@ -377,37 +377,42 @@ class EPBuffer(BufferBase):
 
         def epilogue():
             # the inputs stay referenced by this closure until the copy kernel has been enqueued
+            per_expert_list: List[int] = []
             if cached_mode:
                 num_recv, num_expanded = cached_num_recv_tokens, cached_num_expanded_tokens
-                per_expert_list: List[int] = cached_num_recv_tokens_per_expert_list
+                per_expert_list = cached_num_recv_tokens_per_expert_list
+                alloc_recv, alloc_expanded = num_recv, num_expanded
             elif do_cpu_sync:
-                c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
-                c_list = (ctypes.c_int * max(1, num_local_experts))()
-                _check(_ep_wait(self._h, ctypes.byref(c_recv), ctypes.byref(c_exp), c_list))
-                num_recv, num_expanded = c_recv.value, c_exp.value
-                per_expert_list = [c_list[i] for i in range(num_local_experts)]
+                # Exact sizes come from the host count page, but waiting for it here would leave the GPU
+                # idle between the layout kernels and the copy.  Allocate for this call's upper bound,
+                # enqueue the copy, and read the counts while it runs; the results are narrowed below.
+                alloc_recv = num_tokens
+                alloc_expanded = num_tokens * min(num_topk, num_local_experts) + (expert_alignment - 1) * num_local_experts
+                alloc_expanded = -(-alloc_expanded // expert_alignment) * expert_alignment
+                num_recv = num_expanded = None
             else:
                 c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
                 _check(_ep_worst(self._h, num_max_tokens_per_rank, num_topk, num_experts, expert_alignment,
                                  ctypes.byref(c_recv), ctypes.byref(c_exp)))
-                num_recv, num_expanded, per_expert_list = c_recv.value, c_exp.value, []
+                num_recv, num_expanded = c_recv.value, c_exp.value
+                alloc_recv, alloc_expanded = num_recv, num_expanded
 
             out_dtype = torch.float8_e4m3fn if fused_fp8_quant else x.dtype
-            recv_x = torch.empty((num_expanded, hidden), dtype=out_dtype, device=dev)
+            recv_x = torch.empty((alloc_expanded, hidden), dtype=out_dtype, device=dev)
             recv_sf = None
             if fused_fp8_quant:
-                recv_sf = torch.empty((num_expanded, (hidden + 127) // 128), dtype=torch.float32, device=dev)
+                recv_sf = torch.empty((alloc_expanded, (hidden + 127) // 128), dtype=torch.float32, device=dev)
             elif sf is not None:
-                recv_sf = torch.empty((num_expanded, sf.size(1)), dtype=sf.dtype, device=dev)
+                recv_sf = torch.empty((alloc_expanded, sf.size(1)), dtype=sf.dtype, device=dev)
             recv_topk_weights = None
             if topk_weights is not None:
-                recv_topk_weights = torch.empty((num_expanded,), dtype=topk_weights.dtype, device=dev)
+                recv_topk_weights = torch.empty((alloc_expanded,), dtype=topk_weights.dtype, device=dev)
             if cached_mode:
                 recv_src_metadata = cached_recv_src_metadata
                 if recv_src_metadata.dim() != 2 or recv_src_metadata.size(0) != num_recv:
                     raise EPException('Assertion exception (_C.py): recv_src_metadata.size(0) == num_recv_tokens')
             else:
-                recv_src_metadata = ints(num_recv, num_topk + 2)
+                recv_src_metadata = ints(alloc_recv, num_topk + 2)
 
             e = _DispatchEpilogueArgs()
             e.x, e.sf, e.topk_weights = _desc(x), _desc(sf, two_byte_packs=True), _desc(topk_weights)
@@ -420,6 +425,19 @@ class EPBuffer(BufferBase):
             e.fused_fp8_quant = int(fused_fp8_quant)
             e.stream = _stream()
             _check(_ep_dispatch_epi(self._h, ctypes.byref(e)))
+
+            if num_recv is None:
+                c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
+                c_list = (ctypes.c_int * max(1, num_local_experts))()
+                _check(_ep_wait(self._h, ctypes.byref(c_recv), ctypes.byref(c_exp), c_list))
+                num_recv, num_expanded = c_recv.value, c_exp.value
+                per_expert_list = [c_list[i] for i in range(num_local_experts)]
+                if num_recv > alloc_recv or num_expanded > alloc_expanded:
+                    raise EPException('Assertion exception (_C.py): received counts exceed this call\'s bound')
+                recv_x = recv_x[:num_expanded]
+                recv_sf = recv_sf[:num_expanded] if recv_sf is not None else None
+                recv_topk_weights = recv_topk_weights[:num_expanded] if recv_topk_weights is not None else None
+                recv_src_metadata = recv_src_metadata[:num_recv]
 
             if recv_sf is not None and use_col_major_sf:
                 recv_sf = recv_sf.transpose(0, 1).contiguous().transpose(0, 1)
