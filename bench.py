@@ -25,6 +25,11 @@ import numpy as np  # noqa: E402
 import torch  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch on the headline workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
+# what the same counter reads for a plain 1 GiB copy (x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE):
+# profiles/headline_dispatch_combine_hbm_traffic.txt.  The scatter figure includes the zero padding.
+MEASURED_TRAFFIC = {('c3_headline', 'ep_scatter_quant'): 241.1e6 + 844.9e6,
+                    ('c3_headline', 'ep_combine_k6'): 1417.1e6 + 235.7e6}
 WORKLOADS = {
     # name: (T, H, E, K, A, fp8)
     'c3_headline': (16384, 7168, 256, 6, 128, True),
@@ -92,8 +97,10 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--workload', default='c3_headline', choices=sorted(WORKLOADS))
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--cpu-sample-tokens', type=int, default=2048)
+    ap.add_argument('--cpu-sample-tokens', type=int, default=16384)
     ap.add_argument('--no-cpu-sync', action='store_true', help='dispatch without the host count wait')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also run a plain 1 GiB device copy (known traffic) to scale rocprof byte counters')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py measures one GPU\'s share of the EP path; run it with --gpus 1 (no collectives exist here)',
@@ -104,6 +111,13 @@ def main():
     T, H, E, K, A, fp8 = WORKLOADS[args.workload]
     dev = torch.device('cuda', 0)
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)          # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     x, topk, w = make_inputs(T, H, E, K)
     xg, tg, wg = x.to(dev), topk.to(dev), w.to(dev)
     buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K,
@@ -161,8 +175,9 @@ def main():
 
     def roof(name, nbytes, us):
         gbs = nbytes / us / 1e3
+        traffic = MEASURED_TRAFFIC.get((args.workload, name)) if not args.no_cpu_sync else None
         return {'kernel': name, 'bound': 'hbm', 'achieved': round(gbs, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': round(gbs / HBM_PEAK_GBS, 4), 'traffic': None, 'us': round(us, 2), 'bytes': nbytes}
+                'frac': round(gbs / HBM_PEAK_GBS, 4), 'traffic': traffic, 'us': round(us, 2), 'bytes': nbytes}
 
     scatter_name = 'ep_scatter_quant' if fp8 else 'ep_scatter_copy'
     kernels = [roof(scatter_name, b_d, us_scatter), roof(f'ep_combine_k{K}', b_c, us_combine)]
