@@ -14,6 +14,14 @@
 #define EP_ROWS_PER_BLOCK 4
 #define EP_PAD_BLOCKS_PER_EXPERT 4
 
+#define EP_SCATTER_EXPAND 0
+#define EP_SCATTER_PACK 1
+#define EP_SCATTER_REGION 2
+
+#define EP_COMBINE_FUSED 0      // single partition: owner-side and token-side reduce in one pass
+#define EP_COMBINE_PARTIAL 1    // owner side: per received row, partial into the combine buffer
+#define EP_COMBINE_FINAL 2      // token side: biases + partials of the masters into combined_x
+
 // Host-visible count page (pinned, mapped).  Written once per non-cached dispatch.
 //   [0] ready sequence number (written last, release at system scope)
 //   [1] number of received tokens   [2] number of expanded tokens (aligned)
@@ -75,6 +83,16 @@ struct EpScatterArgs {
     int num_row_blocks;           // blocks [0, num_row_blocks) copy rows, the rest zero padding
     int num_tokens;               // T: bound of the token indices a row may name
     int num_parts;                // column parts per row; a wave task is (row, part)
+    int mode;                     // EP_SCATTER_*
+    // partitioned path (EP_SCATTER_PACK / EP_SCATTER_REGION)
+    const int64_t* topk_idx;      // [T, K]            (pack)
+    const int* dst_slot_idx;      // [T, K]            (pack)
+    int64_t copy_bytes;           // payload bytes moved per row (verbatim kernel)
+    int64_t src_base_row;         // first packed row of this partition's own region (region mode)
+    int num_experts, experts_per_rank;
+    int with_metadata;            // packed rows carry topk_idx and the source token (non-cached)
+    int idx_off, w_off, src_off;  // byte offsets of the packed metadata inside a row
+    int num_out_rows;             // rows of recv_x: slots outside are ignored
     int pad0;
 };
 
@@ -95,6 +113,11 @@ struct EpCombineArgs {
     int num_row_blocks;           // blocks [0, num_row_blocks) reduce rows, the rest handle unrouted tokens
     int num_experts;
     int num_parts;                // 1024-channel parts per row; a wave task is (row, part)
+    int64_t y_row_bytes;          // stride of the rows being gathered (hidden*2, or a combine-buffer token)
+    int64_t out_row_bytes;        // stride of the rows being written
+    int num_ranks, experts_per_rank;
+    int num_in_rows;              // rows of y: slots outside are ignored
+    int num_groups;               // partial groups of the combine buffer: min(K, R)
 };
 
 // Hardware vs integer e4m3fn conversion over fp32 bit patterns [first, first+count).

@@ -319,16 +319,52 @@ __device__ __forceinline__ u32x2 quant8(const float* f, float inv) {
 }
 
 struct RowCtx {
-    int t;        // local token index of the row
-    int myslot;   // lane j < K: expanded slot of (row, j) or -1
+    int t;            // local token index of the row
+    int myslot;       // lane j < K: destination row of (row, j) or -1
+    int64_t src_row;  // row of the source matrix holding the payload
 };
 
-// A wave task is (receive-stream row, column part).  Resolves the row's token and slots; the task
-// of part 0 also writes (non-cached) the metadata row and scatters the gate weights.
+// A wave task is (row, column part).  Resolves the row's token, its source row and its destination
+// rows; the task of part 0 also writes the row's small items.  Three modes:
+//   EP_SCATTER_EXPAND  rows of the receive stream, payload read from x[token]; destinations are the
+//                      expanded slots; part 0 writes the metadata row (non-cached) and the gate weights
+//   EP_SCATTER_PACK    rows are tokens; destinations are rows of the partition-major regions
+//                      (partition * max_tokens + slot of dst_buffer_slot_idx); part 0 writes the packed
+//                      metadata [all K topk_idx | all K weights | src_token_global_idx] into each of them
+//                      (impls/ep/dispatch.hpp:768-794, layout/ep/token.hpp:59-82)
+//   EP_SCATTER_REGION  rows of the receive stream, payload, scales and weights read from the packed rows
+//                      of this partition's own region (dispatch_copy_epilogue.hpp:459-522)
 __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int i, int part, RowCtx& c) {
     const int lane = lane_id();
     const int K = a.num_topk;
     int myslot = -1, t;
+    if (a.mode == EP_SCATTER_PACK) {
+        t = i;
+        int64_t e = -1;
+        if (lane < K) {
+            e = a.topk_idx[(int64_t)t * K + lane];
+            const int s = a.dst_slot_idx[(int64_t)t * K + lane];
+            if (s >= 0 && s < a.max_tokens && e >= 0 && e < a.num_experts)
+                myslot = (int)(e / a.experts_per_rank) * a.max_tokens + s;
+        }
+        if (part == 0) {
+            const float w = (a.topk_weights != nullptr && lane < K) ? a.topk_weights[(int64_t)t * K + lane] : 0.0f;
+            for (int j = 0; j < K; ++j) {
+                const int g = readlane(myslot, j);
+                if (g < 0) continue;
+                char* row = (char*)a.recv_x + (int64_t)g * a.out_row_bytes;
+                if (lane < K) {
+                    if (a.with_metadata) ((int64_t*)(row + a.idx_off))[lane] = e;
+                    ((float*)(row + a.w_off))[lane] = w;
+                }
+                if (a.with_metadata && lane == 0) *(int*)(row + a.src_off) = a.rank_idx * a.max_tokens + t;
+            }
+        }
+        c.t = t;
+        c.myslot = myslot;
+        c.src_row = t;
+        return true;
+    }
     if (!a.cached) {
         t = a.recv_tok[i];
         if (t < 0 || t >= a.num_tokens) return false;
@@ -346,8 +382,14 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
         t = readlane(v, K) - a.rank_idx * a.max_tokens;
         if (t < 0 || t >= a.num_tokens) return false;
     }
-    if (part == 0 && a.recv_topk_weights != nullptr && lane < K && myslot >= 0)
-        a.recv_topk_weights[myslot] = a.topk_weights[(int64_t)t * K + lane];
+    if (lane < K && (myslot < 0 || myslot >= a.num_out_rows)) myslot = -1;
+    c.src_row = a.mode == EP_SCATTER_REGION ? a.src_base_row + i : (int64_t)t;
+    if (part == 0 && a.recv_topk_weights != nullptr && lane < K && myslot >= 0) {
+        const float* w = a.mode == EP_SCATTER_REGION
+            ? (const float*)((const char*)a.x + c.src_row * a.x_row_bytes + a.w_off)
+            : a.topk_weights + (int64_t)t * K;
+        a.recv_topk_weights[myslot] = w[lane];
+    }
     c.t = t;
     c.myslot = myslot;
     return true;
@@ -384,15 +426,15 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
     const int lane = lane_id();
     const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
     const int i = task / a.num_parts, part = task - i * a.num_parts;
-    const int n = min(*a.num_recv_ptr, a.num_rows_bound);
+    const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
     if (i >= n) return;
     RowCtx c;
     if (!scatter_row_prologue(a, i, part, c)) return;
     const int K = a.num_topk;
-    const int nvec = (int)(a.x_row_bytes >> 4);
+    const int nvec = (int)(a.copy_bytes >> 4);
     const int v = part * WAVE + lane;
     if (v < nvec) {
-        const u32x4 d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + (int64_t)c.t * a.x_row_bytes) + v);
+        const u32x4 d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
         for (int j = 0; j < K; ++j) {
             const int s = readlane(c.myslot, j);
             if (s < 0) continue;
@@ -401,7 +443,7 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
     }
     if (part == 0 && a.recv_sf != nullptr) {
         const int P = a.num_sf_packs;
-        const char* sfrow = (const char*)a.sf + (int64_t)c.t * a.sf_token_stride_bytes;
+        const char* sfrow = (const char*)a.sf + c.src_row * a.sf_token_stride_bytes;
         for (int p = lane; p < P; p += WAVE) {
             const unsigned short val = *(const unsigned short*)(sfrow + (int64_t)p * a.sf_pack_stride_bytes);
             for (int j = 0; j < K; ++j) {
@@ -425,7 +467,7 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     const int lane = lane_id();
     const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
     const int i = task / a.num_parts, part = task - i * a.num_parts;
-    const int n = min(*a.num_recv_ptr, a.num_rows_bound);
+    const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
     if (i >= n) return;
     RowCtx c;
     if (!scatter_row_prologue(a, i, part, c)) return;
@@ -434,7 +476,7 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     const int v = part * WAVE + lane;
     const bool live = v < nvec;
     u32x4 d = {0u, 0u, 0u, 0u};
-    if (live) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + (int64_t)c.t * a.x_row_bytes) + v);
+    if (live) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
     float f[8] = {bf16_lo(d.x), bf16_hi(d.x), bf16_lo(d.y), bf16_hi(d.y),
                   bf16_lo(d.z), bf16_hi(d.z), bf16_lo(d.w), bf16_hi(d.w)};
     float m = 0.0f;
@@ -543,11 +585,20 @@ __device__ __forceinline__ void combine_unrouted(const EpCombineArgs& a) {
     }
 }
 
-// A wave task is (receive-stream row, 1024-channel part): two 16-byte vectors per lane and slot,
-// all K*2 loads issued before the first add.
-template <int KT>
+// A wave task is (row, 1024-channel part): two 16-byte vectors per lane and input row, all loads
+// issued before the first add.  MODE selects which reduction of the reference the task performs:
+//   EP_COMBINE_FUSED    one partition: rows are the receive stream; out = BF16(sum_j f32 y[slot_j]), then
+//                       BF16(f32 b0 + f32 b1 + f32 that) when biases are given (the two levels of
+//                       combine.hpp:291-324 and combine_reduce_epilogue.hpp:114-140 for a single master)
+//   EP_COMBINE_PARTIAL  owner side: same sum, stored with its K-wide weight vector in the combine buffer
+//                       at [group * max_tokens + source token]            (combine.hpp:94-106,301-324)
+//   EP_COMBINE_FINAL    token side: rows are tokens; inputs = b0, b1, then the partial of every master
+//                       (last top-k position per destination partition) in ascending position, summed
+//                       left to right in fp32 and rounded once; weight vectors OR-merged
+//                       (combine_reduce_epilogue.hpp:96-153)
+template <int KT, int MODE>
 __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
-    if ((int)blockIdx.x >= a.num_row_blocks) {
+    if (MODE == EP_COMBINE_FUSED && (int)blockIdx.x >= a.num_row_blocks) {
         combine_unrouted(a);
         return;
     }
@@ -555,36 +606,94 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     const int K = KT > 0 ? KT : a.num_topk;
     const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
     const int i = task / a.num_parts, part = task - i * a.num_parts;
-    const int n = min(*a.num_recv_ptr, a.num_rows_bound);
+    const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
     if (i >= n) return;
-    const int mv = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
-    const int myslot = lane < K ? mv : -1;
-    const int t = readlane(mv, K) - a.rank_idx * a.max_tokens;
-    if (t < 0 || t >= a.num_tokens) return;
+
+    int myslot = -1, t, group = 0;
+    if (MODE == EP_COMBINE_FINAL) {
+        t = i;
+        int r = -1;
+        if (lane < K) {
+            const int64_t e = a.topk_idx[(int64_t)t * K + lane];
+            if (e >= 0 && e < a.num_experts) r = (int)(e / a.experts_per_rank);
+        }
+        bool master = r >= 0;
+        for (int jj = 1; jj < K; ++jj) {
+            const int rj = readlane(r, jj);
+            if (lane < jj && rj == r) master = false;          // a later position goes to the same partition
+        }
+        if (master) myslot = (a.num_ranks < K ? r : lane) * a.max_tokens + t;
+    } else {
+        const int mv = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
+        if (lane < K && mv >= 0 && mv < a.num_in_rows) myslot = mv;
+        t = readlane(mv, K) - a.rank_idx * a.max_tokens;
+        if (t < 0 || t >= a.max_tokens) return;
+        if (MODE == EP_COMBINE_FUSED && t >= a.num_tokens) return;
+        group = a.num_ranks < K ? a.rank_idx : readlane(mv, K + 1);
+        if (MODE == EP_COMBINE_PARTIAL && (group < 0 || group >= a.num_groups)) return;
+    }
     const int nvalid = __popcll(__ballot(myslot >= 0));
-    float myw = 0.0f;
-    if (a.expanded_weights != nullptr && myslot >= 0) myw = a.expanded_weights[myslot];
-    if (part == 0 && a.combined_topk_weights != nullptr && lane < K)
-        a.combined_topk_weights[(int64_t)t * K + lane] = myw;
     const int nvec = a.hidden >> 3;
-    const int64_t rowvec = nvec;
+    const int64_t yvec = a.y_row_bytes >> 4;
     const u32x4* y = (const u32x4*)a.y;
-    u32x4* out = (u32x4*)a.combined_x + (int64_t)t * rowvec;
+    char* out_row = (char*)a.combined_x +
+        (MODE == EP_COMBINE_PARTIAL ? ((int64_t)group * a.max_tokens + t) : (int64_t)t) * a.out_row_bytes;
+
+    // ---- gate weights ----
+    float myw = 0.0f;
+    if (MODE == EP_COMBINE_FINAL) {
+        if (part == 0 && a.combined_topk_weights != nullptr) {
+            unsigned acc = 0;
+            for (int j = 0; j < K; ++j) {
+                const int s = readlane(myslot, j);
+                if (s < 0) continue;
+                if (lane < K) acc |= ((const unsigned*)((const char*)a.y + (int64_t)s * a.y_row_bytes + (a.hidden << 1)))[lane];
+            }
+            if (lane < K) ((unsigned*)a.combined_topk_weights)[(int64_t)t * K + lane] = acc;
+        }
+    } else {
+        if (a.expanded_weights != nullptr && myslot >= 0) myw = a.expanded_weights[myslot];
+        if (part == 0 && lane < K) {
+            if (MODE == EP_COMBINE_FUSED && a.combined_topk_weights != nullptr)
+                a.combined_topk_weights[(int64_t)t * K + lane] = myw;
+            if (MODE == EP_COMBINE_PARTIAL && a.expanded_weights != nullptr)
+                ((float*)(out_row + (a.hidden << 1)))[lane] = myw;
+        }
+    }
+
+    u32x4* out = (u32x4*)out_row;
     const bool has_bias = a.bias_0 != nullptr || a.bias_1 != nullptr;
     const int v0 = part * 2 * WAVE + lane, v1 = v0 + WAVE;
     const bool live0 = v0 < nvec, live1 = v1 < nvec;
     float acc0[8], acc1[8];
     u32x4 res0 = {0u, 0u, 0u, 0u}, res1 = {0u, 0u, 0u, 0u};
+    int nin = 0;                                              // inputs accumulated so far
+    if (MODE == EP_COMBINE_FINAL) {
+        const void* biases[2] = {a.bias_0, a.bias_1};
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            if (biases[b] == nullptr) continue;
+            const u32x4* bp = (const u32x4*)biases[b] + (int64_t)t * nvec;
+            u32x4 e0 = {0u, 0u, 0u, 0u}, e1 = {0u, 0u, 0u, 0u};
+            if (live0) e0 = bp[v0];
+            if (live1) e1 = bp[v1];
+            float g0[8], g1[8];
+            unpack8(e0, g0);
+            unpack8(e1, g1);
+            if (nin == 0) { for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; } res0 = e0; res1 = e1; }
+            else { for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; } }
+            ++nin;
+        }
+    }
     if (KT > 0) {
         u32x4 d0[KT > 0 ? KT : 1], d1[KT > 0 ? KT : 1];
 #pragma unroll
         for (int j = 0; j < KT; ++j) {
             const int s = readlane(myslot, j);
             if (s < 0) continue;
-            if (live0) d0[j] = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v0);
-            if (live1) d1[j] = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v1);
+            if (live0) d0[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + v0);
+            if (live1) d1[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + v1);
         }
-        bool first = true;
 #pragma unroll
         for (int j = 0; j < KT; ++j) {
             const int s = readlane(myslot, j);
@@ -592,61 +701,58 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
             float g0[8], g1[8];
             unpack8(d0[j], g0);
             unpack8(d1[j], g1);
-            if (a.weighted) {
+            if (MODE == EP_COMBINE_FUSED && a.weighted) {
                 const float wj = __int_as_float(readlane(__float_as_int(myw), j));
                 for (int q = 0; q < 8; ++q) { g0[q] = g0[q] * wj; g1[q] = g1[q] * wj; }
             }
-            if (first) {
-                for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; }
-                res0 = d0[j]; res1 = d1[j];
-                first = false;
-            } else {
-                for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; }
-            }
+            if (nin == 0) { for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; } res0 = d0[j]; res1 = d1[j]; }
+            else { for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; } }
+            ++nin;
         }
     } else {
-        bool first = true;
         for (int j = 0; j < K; ++j) {
             const int s = readlane(myslot, j);
             if (s < 0) continue;
             u32x4 e0 = {0u, 0u, 0u, 0u}, e1 = {0u, 0u, 0u, 0u};
-            if (live0) e0 = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v0);
-            if (live1) e1 = __builtin_nontemporal_load(y + (int64_t)s * rowvec + v1);
+            if (live0) e0 = __builtin_nontemporal_load(y + (int64_t)s * yvec + v0);
+            if (live1) e1 = __builtin_nontemporal_load(y + (int64_t)s * yvec + v1);
             float g0[8], g1[8];
             unpack8(e0, g0);
             unpack8(e1, g1);
-            if (a.weighted) {
+            if (MODE == EP_COMBINE_FUSED && a.weighted) {
                 const float wj = __int_as_float(readlane(__float_as_int(myw), j));
                 for (int q = 0; q < 8; ++q) { g0[q] = g0[q] * wj; g1[q] = g1[q] * wj; }
             }
-            if (first) {
-                for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; }
-                res0 = e0; res1 = e1;
-                first = false;
-            } else {
-                for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; }
-            }
+            if (nin == 0) { for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; } res0 = e0; res1 = e1; }
+            else { for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; } }
+            ++nin;
         }
     }
-    if (nvalid >= 2 || (a.weighted && nvalid == 1)) {
+    // zero inputs -> zeros, one input -> verbatim copy, more -> one rounding of the fp32 sum
+    if (nin >= 2 || (MODE == EP_COMBINE_FUSED && a.weighted && nvalid == 1)) {
         res0 = pack8(acc0);
         res1 = pack8(acc1);
     }
     if (live0) {
-        if (has_bias) res0 = add_biases(a, t, v0, true, res0);
+        if (MODE == EP_COMBINE_FUSED && has_bias) res0 = add_biases(a, t, v0, true, res0);
         __builtin_nontemporal_store(res0, out + v0);
     }
     if (live1) {
-        if (has_bias) res1 = add_biases(a, t, v1, true, res1);
+        if (MODE == EP_COMBINE_FUSED && has_bias) res1 = add_biases(a, t, v1, true, res1);
         __builtin_nontemporal_store(res1, out + v1);
     }
 }
 
-extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_generic(EpCombineArgs a) { combine_body<0>(a); }
-extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_k2(EpCombineArgs a) { combine_body<2>(a); }
-extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_k4(EpCombineArgs a) { combine_body<4>(a); }
-extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_k6(EpCombineArgs a) { combine_body<6>(a); }
-extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine_k8(EpCombineArgs a) { combine_body<8>(a); }
+#define EP_COMBINE_KERNELS(SUFFIX, MODE)                                                                                   \
+    extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine##SUFFIX##_generic(EpCombineArgs a) { combine_body<0, MODE>(a); } \
+    extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine##SUFFIX##_k2(EpCombineArgs a) { combine_body<2, MODE>(a); }     \
+    extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine##SUFFIX##_k4(EpCombineArgs a) { combine_body<4, MODE>(a); }     \
+    extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine##SUFFIX##_k6(EpCombineArgs a) { combine_body<6, MODE>(a); }     \
+    extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_combine##SUFFIX##_k8(EpCombineArgs a) { combine_body<8, MODE>(a); }
+
+EP_COMBINE_KERNELS(, EP_COMBINE_FUSED)
+EP_COMBINE_KERNELS(_partial, EP_COMBINE_PARTIAL)
+EP_COMBINE_KERNELS(_final, EP_COMBINE_FINAL)
 
 // ------------------------------------------------------------------------------------------------
 // Self-test: hardware e4m3fn conversion against the integer conversion over a range of fp32 bit

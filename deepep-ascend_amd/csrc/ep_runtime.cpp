@@ -81,6 +81,22 @@ int64_t token_bytes(int hidden_bytes, int sf_bytes, int topk, bool with_metadata
     return n + align_up(meta, kUbAlign);
 }
 
+// Byte offsets inside a packed token (reference: layout/ep/token.hpp:59-82).
+struct PackedToken {
+    int64_t bytes;
+    int sf_off, idx_off, w_off, src_off;
+};
+
+PackedToken packed_token(int hidden_bytes, int sf_bytes, int topk, bool with_metadata) {
+    PackedToken p{};
+    p.bytes = token_bytes(hidden_bytes, sf_bytes, topk, with_metadata);
+    p.sf_off = (int)align_up(hidden_bytes, kUbAlign);
+    p.idx_off = sf_bytes > 0 ? p.sf_off + (int)align_up(sf_bytes, kUbAlign) : hidden_bytes;
+    p.w_off = p.idx_off + (with_metadata ? (int)align_up((int64_t)topk * 8, kUbAlign) : 0);
+    p.src_off = p.w_off + topk * 4;
+    return p;
+}
+
 int64_t dispatch_buffer_size(int max_tokens, int hidden, int sf_packs, int topk, int elem, int ranks) {
     return (int64_t)ranks * max_tokens * token_bytes(hidden * elem, sf_packs * 2, topk, true);
 }
@@ -94,7 +110,7 @@ struct Kernels {
     hipModule_t module = nullptr;
     hipFunction_t layout_count, layout_scan, layout_assign;
     hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw;
-    hipFunction_t combine_generic, combine_k2, combine_k4, combine_k6, combine_k8;
+    hipFunction_t combine[3][5];     // [mode][generic, k2, k4, k6, k8]
     hipFunction_t fp8_selftest;
     int device = -1;
 };
@@ -131,11 +147,11 @@ void load_kernels(const char* dir) {
     get(g_k.scatter_copy, "ep_scatter_copy");
     get(g_k.scatter_quant, "ep_scatter_quant");
     get(g_k.scatter_quant_sw, "ep_scatter_quant_sw");
-    get(g_k.combine_generic, "ep_combine_generic");
-    get(g_k.combine_k2, "ep_combine_k2");
-    get(g_k.combine_k4, "ep_combine_k4");
-    get(g_k.combine_k6, "ep_combine_k6");
-    get(g_k.combine_k8, "ep_combine_k8");
+    const char* modes[3] = {"", "_partial", "_final"};
+    const char* ks[5] = {"_generic", "_k2", "_k4", "_k6", "_k8"};
+    for (int mode = 0; mode < 3; ++mode)
+        for (int k = 0; k < 5; ++k)
+            get(g_k.combine[mode][k], (std::string("ep_combine") + modes[mode] + ks[k]).c_str());
     get(g_k.fp8_selftest, "ep_fp8_selftest");
     g_k.module = m;
 }
@@ -427,9 +443,51 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         EP_HOST_ASSERT(unaligned.dtype == EP_DTYPE_I32);
         EP_HOST_ASSERT(a.dst_buffer_slot_idx.dtype == EP_DTYPE_I32 and a.dst_gsge_idx.dtype == EP_DTYPE_I32);
 
+        // geometry of the packed rows of the partition-major regions (only materialised when R > 1)
+        const PackedToken pk = packed_token(hidden * packed_elem, packed_sf * 2, num_topk, not cached_mode);
+        auto launch_pack = [&]() {
+            EpScatterArgs sa{};
+            sa.mode = EP_SCATTER_PACK;
+            sa.x = a.x.data;
+            sa.sf = a.sf.data;
+            sa.topk_weights = (const float*)a.topk_weights.data;
+            sa.topk_idx = (const int64_t*)a.topk_idx.data;
+            sa.dst_slot_idx = (const int*)a.dst_buffer_slot_idx.data;
+            sa.recv_x = b->buffer();
+            sa.recv_sf = packed_sf > 0 ? b->buffer() + pk.sf_off : nullptr;
+            sa.x_row_bytes = (int64_t)hidden * x_elem;
+            sa.copy_bytes = sa.x_row_bytes;
+            sa.out_row_bytes = pk.bytes;
+            sa.out_sf_row_bytes = pk.bytes;
+            if (present(a.sf)) {
+                sa.sf_token_stride_bytes = a.sf.stride[0] * 2;
+                sa.sf_pack_stride_bytes = a.sf.stride[1] * 2;
+            }
+            sa.hidden = hidden;
+            sa.num_topk = num_topk;
+            sa.num_rows_bound = num_tokens;
+            sa.num_tokens = num_tokens;
+            sa.rank_idx = b->rank_idx;
+            sa.max_tokens = a.num_max_tokens_per_rank;
+            sa.num_sf_packs = num_sf_packs;
+            sa.num_experts = a.num_experts;
+            sa.experts_per_rank = num_experts_per_rank;
+            sa.with_metadata = cached_mode ? 0 : 1;
+            sa.idx_off = pk.idx_off;
+            sa.w_off = pk.w_off;
+            sa.src_off = pk.src_off;
+            sa.num_out_rows = num_ranks * a.num_max_tokens_per_rank;
+            sa.num_parts = (int)std::max<int64_t>(1, a.fused_fp8_quant ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024));
+            sa.num_row_blocks = (int)ceil_div((int64_t)num_tokens * sa.num_parts, EP_ROWS_PER_BLOCK);
+            if (sa.num_row_blocks == 0) return;
+            hipFunction_t fn = a.fused_fp8_quant ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
+            launch(fn, (unsigned)sa.num_row_blocks, EP_ROW_THREADS, 0, a.stream, sa);
+        };
+
         if (cached_mode) {
-            // the cached handle already holds the whole layout: nothing to enqueue before the epilogue
+            // the cached handle already holds the whole layout: only the packed regions are refreshed
             b->last.valid = false;
+            if (num_ranks > 1) launch_pack();
             return;
         }
 
@@ -481,6 +539,8 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, smem_count, a.stream, la);
         launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 64), EP_SCAN_THREADS, 0, a.stream, la);
         launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, a.stream, la);
+
+        if (num_ranks > 1) launch_pack();
 
         b->last.valid = true;
         b->last.num_tokens = num_tokens;
@@ -542,8 +602,6 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         EP_HOST_ASSERT(a.num_experts % R == 0);
         const int El = a.num_experts / R;
         const bool fused = a.fused_fp8_quant != 0;
-        EP_HOST_ASSERT(R == 1 and "partitioned receive is launched through the packed-region path");
-
         EP_HOST_ASSERT(present(a.recv_x) and a.recv_x.ndim == 2 and a.recv_x.size[1] == hidden);
         EP_HOST_ASSERT(contiguous(a.recv_x));
         EP_HOST_ASSERT(a.recv_x.dtype == (fused ? (int)EP_DTYPE_FP8_E4M3 : a.x.dtype));
@@ -578,8 +636,6 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         }
 
         EpScatterArgs sa{};
-        sa.x = a.x.data;
-        sa.sf = a.sf.data;
         sa.topk_weights = (const float*)a.topk_weights.data;
         sa.slot_map = b->last.slot_map;
         sa.recv_tok = b->last.recv_tok;
@@ -589,12 +645,7 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.recv_sf = has_sf ? a.recv_sf.data : nullptr;
         sa.recv_topk_weights = present(a.topk_weights) ? (float*)a.recv_topk_weights.data : nullptr;
         sa.psum_expert = (const int*)a.psum_num_recv_tokens_per_expert.data;
-        sa.x_row_bytes = (int64_t)hidden * elem_size(a.x.dtype);
         sa.out_row_bytes = (int64_t)hidden * elem_size(a.recv_x.dtype);
-        if (present(a.sf)) {
-            sa.sf_token_stride_bytes = a.sf.stride[0] * 2;
-            sa.sf_pack_stride_bytes = a.sf.stride[1] * 2;
-        }
         sa.out_sf_row_bytes = has_sf ? a.recv_sf.size[1] * elem_size(a.recv_sf.dtype) : 0;
         sa.hidden = hidden;
         sa.num_topk = K;
@@ -604,18 +655,49 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.rank_idx = b->rank_idx;
         sa.max_tokens = a.num_max_tokens_per_rank;
         sa.cached = cached_mode ? 1 : 0;
-        sa.num_sf_packs = num_sf_packs;
         sa.num_local_experts = El;
         sa.expert_alignment = a.expert_alignment;
         sa.zero_padding = a.do_zero_padding ? 1 : 0;
+        sa.num_out_rows = (int)std::min<int64_t>(num_expanded, INT32_MAX);
+        bool quantise_here = fused;
+        if (R == 1) {
+            // one partition: the packed intermediate is skipped, rows come straight from x
+            sa.mode = EP_SCATTER_EXPAND;
+            sa.x = a.x.data;
+            sa.sf = a.sf.data;
+            sa.x_row_bytes = (int64_t)hidden * elem_size(a.x.dtype);
+            sa.copy_bytes = sa.x_row_bytes;
+            if (present(a.sf)) {
+                sa.sf_token_stride_bytes = a.sf.stride[0] * 2;
+                sa.sf_pack_stride_bytes = a.sf.stride[1] * 2;
+            }
+            sa.num_sf_packs = num_sf_packs;
+        } else {
+            // expand this partition's own region of the packed rows written by ep_dispatch_launch
+            const int payload_elem = fused ? 1 : elem_size(a.x.dtype);
+            const int sf_packs = fused ? 2 * (int)ceil_div(hidden, 128) : num_sf_packs;
+            const PackedToken pk = packed_token(hidden * payload_elem, sf_packs * 2, K, not cached_mode);
+            EP_HOST_ASSERT((int64_t)R * a.num_max_tokens_per_rank * pk.bytes <= b->num_buffer_bytes);
+            sa.mode = EP_SCATTER_REGION;
+            sa.x = b->buffer();
+            sa.x_row_bytes = pk.bytes;
+            sa.copy_bytes = (int64_t)hidden * payload_elem;
+            sa.src_base_row = (int64_t)b->rank_idx * a.num_max_tokens_per_rank;
+            sa.sf = sf_packs > 0 ? b->buffer() + pk.sf_off : nullptr;
+            sa.sf_token_stride_bytes = pk.bytes;
+            sa.sf_pack_stride_bytes = 2;
+            sa.num_sf_packs = sf_packs;
+            sa.w_off = pk.w_off;
+            quantise_here = false;
+        }
         // a wave task covers 1 KiB of a verbatim row, or 512 channels of a row being quantised
-        sa.num_parts = (int)std::max<int64_t>(1, fused ? ceil_div(hidden, 512) : ceil_div(sa.x_row_bytes, 1024));
+        sa.num_parts = (int)std::max<int64_t>(1, quantise_here ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024));
         sa.num_row_blocks = (int)ceil_div((int64_t)sa.num_rows_bound * sa.num_parts, EP_ROWS_PER_BLOCK);
         EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0);
         const unsigned pad_blocks = a.do_zero_padding ? (unsigned)El * EP_PAD_BLOCKS_PER_EXPERT : 0u;
         const unsigned grid = (unsigned)sa.num_row_blocks + pad_blocks;
         if (grid == 0) return;
-        hipFunction_t fn = fused ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
+        hipFunction_t fn = quantise_here ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
         launch(fn, grid, EP_ROW_THREADS, 0, a.stream, sa);
     });
 }
@@ -670,8 +752,40 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
         }
         EP_HOST_ASSERT(combine_buffer_size(R, a.num_max_tokens_per_rank, hidden, K) <= b->num_buffer_bytes);
         EP_HOST_ASSERT(phase == 0 or phase == 1);
-        EP_HOST_ASSERT(R == 1 and "partitioned combine is launched through the packed-region path");
-        if (phase == 0) return;     // single partition: the whole reduction is one token-side launch
+        EP_HOST_ASSERT(not a.apply_weights or R == 1);
+        const int kidx = K == 2 ? 1 : K == 4 ? 2 : K == 6 ? 3 : K == 8 ? 4 : 0;
+        const int64_t combine_token = token_bytes(hidden * 2, 0, K, false);
+
+        EpCombineArgs ca{};
+        ca.expanded_weights = (const float*)a.topk_weights.data;
+        ca.recv_src_metadata = (const int*)a.src_metadata.data;
+        ca.topk_idx = (const int64_t*)a.combined_topk_idx.data;
+        ca.hidden = hidden;
+        ca.num_topk = K;
+        ca.num_tokens = num_combined_tokens;
+        ca.rank_idx = b->rank_idx;
+        ca.max_tokens = a.num_max_tokens_per_rank;
+        ca.num_parts = (int)std::max<int64_t>(1, ceil_div(hidden, 1024));
+        ca.num_experts = a.num_experts;
+        ca.num_ranks = R;
+        ca.experts_per_rank = a.num_experts / R;
+        ca.num_groups = std::min(K, R);
+
+        if (phase == 0) {
+            if (R == 1) return;     // single partition: the whole reduction is one token-side launch
+            // owner side: one partial per received row into this GPU's combine buffer
+            ca.y = a.x.data;
+            ca.y_row_bytes = (int64_t)hidden * 2;
+            ca.num_in_rows = num_tokens;
+            ca.num_recv_ptr = (const int*)psum_rank.data + (R - 1);
+            ca.num_rows_bound = (int)a.src_metadata.size[0];
+            ca.combined_x = b->buffer();
+            ca.out_row_bytes = combine_token;
+            ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
+            if (ca.num_row_blocks == 0) return;
+            launch(g_k.combine[EP_COMBINE_PARTIAL][kidx], (unsigned)ca.num_row_blocks, EP_ROW_THREADS, 0, a.stream, ca);
+            return;
+        }
 
         EP_HOST_ASSERT(present(a.combined_x) and a.combined_x.ndim == 2);
         EP_HOST_ASSERT(a.combined_x.size[0] == num_combined_tokens and a.combined_x.size[1] == hidden);
@@ -681,38 +795,33 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             EP_HOST_ASSERT(present(w) and w.ndim == 2 and w.size[0] == num_combined_tokens and w.size[1] == K);
             EP_HOST_ASSERT(contiguous(w) and w.dtype == EP_DTYPE_F32);
         }
-
-        EpCombineArgs ca{};
-        ca.y = a.x.data;
-        ca.expanded_weights = (const float*)a.topk_weights.data;
         ca.bias_0 = a.bias_0.data;
         ca.bias_1 = a.bias_1.data;
-        ca.recv_src_metadata = (const int*)a.src_metadata.data;
-        ca.num_recv_ptr = (const int*)psum_rank.data + (R - 1);
-        ca.topk_idx = (const int64_t*)a.combined_topk_idx.data;
         ca.combined_x = a.combined_x.data;
         ca.combined_topk_weights = present(a.topk_weights) ? (float*)a.combined_topk_weights.data : nullptr;
-        ca.hidden = hidden;
-        ca.num_topk = K;
-        ca.num_tokens = num_combined_tokens;
-        ca.num_rows_bound = (int)a.src_metadata.size[0];
-        ca.rank_idx = b->rank_idx;
-        ca.max_tokens = a.num_max_tokens_per_rank;
-        ca.weighted = a.apply_weights ? 1 : 0;
-        ca.num_parts = (int)std::max<int64_t>(1, ceil_div(hidden, 1024));
-        ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
-        ca.num_experts = a.num_experts;
-        const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(num_combined_tokens, EP_ROW_THREADS);
-        if (grid == 0) return;
-        hipFunction_t fn = g_k.combine_generic;
-        switch (K) {
-            case 2: fn = g_k.combine_k2; break;
-            case 4: fn = g_k.combine_k4; break;
-            case 6: fn = g_k.combine_k6; break;
-            case 8: fn = g_k.combine_k8; break;
-            default: break;
+        ca.out_row_bytes = (int64_t)hidden * 2;
+        if (R == 1) {
+            ca.y = a.x.data;
+            ca.y_row_bytes = (int64_t)hidden * 2;
+            ca.num_in_rows = num_tokens;
+            ca.num_recv_ptr = (const int*)psum_rank.data + (R - 1);
+            ca.num_rows_bound = (int)a.src_metadata.size[0];
+            ca.weighted = a.apply_weights ? 1 : 0;
+            ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
+            const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(num_combined_tokens, EP_ROW_THREADS);
+            if (grid == 0) return;
+            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, 0, a.stream, ca);
+        } else {
+            // token side: biases + the partial of every master, read from the combine buffer
+            ca.y = b->buffer();
+            ca.y_row_bytes = combine_token;
+            ca.num_in_rows = ca.num_groups * a.num_max_tokens_per_rank;
+            ca.num_recv_ptr = nullptr;
+            ca.num_rows_bound = num_combined_tokens;
+            ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROW_THREADS / 64);
+            if (ca.num_row_blocks == 0) return;
+            launch(g_k.combine[EP_COMBINE_FINAL][kidx], (unsigned)ca.num_row_blocks, EP_ROW_THREADS, 0, a.stream, ca);
         }
-        launch(fn, grid, EP_ROW_THREADS, 0, a.stream, ca);
     });
 }
 

@@ -315,6 +315,14 @@ class EPBuffer(BufferBase):
         ptr = _ep_region(self._h, which, ctypes.byref(n))
         return ptr, n.value
 
+    def buffer_tensor(self) -> torch.Tensor:
+        """The communication buffer of the arena (partition-major packed rows after a dispatch with more
+        than one partition, the combine buffer of partials during a combine) as a uint8 tensor."""
+        ptr, n = self.region(1)
+        if n == 0:
+            return torch.empty(0, dtype=torch.uint8, device=self.device)
+        return torch.as_tensor(_DevicePointer(ptr, n, self), device=self.device)
+
     def lb_prefetch_weights(self, *args, **kwargs):
         raise EPException('Assertion exception: EPBuffer::lb_prefetch_weights is not implemented')
 
