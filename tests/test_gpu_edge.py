@@ -1,0 +1,217 @@
+"""Edge cases of the dispatch/combine path: empty and fully masked inputs, ragged sizes, odd top-k and
+hidden sizes, stream/lifetime behaviour under allocator reuse, running statistics, handle guards."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_bits, make_routing, make_tokens
+from oracle import ep_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def _buffer(maxT, H, K, R=1, rank=0, **kw):
+    import deep_ep
+    return deep_ep.EPBuffer(deep_ep.LocalGroup(rank, R), num_max_tokens_per_rank=maxT, hidden=H, num_topk=K,
+                            explicitly_destroy=True, **kw)
+
+
+def _roundtrip(T, maxT, H, E, K, A, topk, w, x, R=1, rank=0, fused=False, seed=0):
+    lay = O.rank_share_layout(topk.numpy(), E, R, rank, A, maxT)
+    buf = _buffer(maxT, H, K, R, rank, use_fp8_dispatch=fused)
+    out = buf.dispatch(x.to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV), num_experts=E,
+                       num_max_tokens_per_rank=maxT, expert_alignment=A, do_expand=True, do_zero_padding=True,
+                       fused_fp8_quant=fused)
+    recv, _, rw, handle, _ = out
+    torch.cuda.synchronize()
+    assert np.array_equal(handle.recv_src_metadata.cpu().numpy(), lay['recv_src_metadata'])
+    assert np.array_equal(handle.dst_buffer_slot_idx.cpu().numpy(), lay['dst_buffer_slot_idx'])
+    assert handle.num_expanded_tokens == lay['num_expanded_tokens']
+    if fused:
+        q, s = O.quantise(x)
+        ex, es, ew = O.rank_share_dispatch(q.numpy(), s.numpy().view(np.uint32), w.numpy(), lay)
+        assert np.array_equal(recv[0].view(torch.uint8).cpu().numpy().reshape(ex.shape), ex)
+        assert np.array_equal(recv[1].cpu().numpy().view(np.uint32).reshape(es.shape), es)
+    else:
+        ex, _, ew = O.rank_share_dispatch(bf16_bits(x).reshape(T, H), None, w.numpy(), lay)
+        assert np.array_equal(bf16_bits(recv).reshape(ex.shape), ex)
+    assert np.array_equal(rw.cpu().numpy().view(np.uint32), ew.view(np.uint32))
+    if R == 1:
+        y = make_tokens(lay['num_expanded_tokens'], H, seed=seed + 1)
+        cx, cw, _ = buf.combine(y.to(DEV), handle, topk_weights=rw)
+        torch.cuda.synchronize()
+        ox, ow = O.combine_fast(y, torch.from_numpy(ew), lay['recv_src_metadata'], T, K)
+        assert np.array_equal(bf16_bits(cx).reshape(T, H), bf16_bits(ox).reshape(T, H))
+        assert torch.equal(cw.cpu(), ow)
+    buf.destroy()
+    return lay
+
+
+def test_empty_input():
+    T, H, E, K = 0, 256, 8, 2
+    x = torch.empty((0, H), dtype=torch.bfloat16)
+    topk = torch.empty((0, K), dtype=torch.int64)
+    w = torch.empty((0, K), dtype=torch.float32)
+    lay = _roundtrip(T, 16, H, E, K, 4, topk, w, x)
+    assert lay['num_recv_tokens'] == 0 and lay['num_expanded_tokens'] == 0
+
+
+def test_every_slot_masked():
+    T, H, E, K = 40, 256, 8, 3
+    x = make_tokens(T, H)
+    topk = torch.full((T, K), -1, dtype=torch.int64)
+    w = torch.zeros((T, K))
+    lay = _roundtrip(T, T, H, E, K, 8, topk, w, x)
+    assert lay['num_recv_tokens'] == 0
+    # combine of an empty receive stream: bias sum, or zeros
+    buf = _buffer(T, H, K)
+    _, _, rw, handle, _ = buf.dispatch(x.to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV), num_experts=E,
+                                       expert_alignment=8, do_expand=True)
+    y = torch.empty((handle.num_expanded_tokens, H), dtype=torch.bfloat16, device=DEV)
+    b0, b1 = make_tokens(T, H, seed=3), make_tokens(T, H, seed=4)
+    cx, cw, _ = buf.combine(y, handle, topk_weights=rw)
+    assert int(cx.count_nonzero()) == 0 and int(cw.count_nonzero()) == 0
+    cx, _, _ = buf.combine(y, handle, bias=b0.to(DEV))
+    assert torch.equal(cx.cpu(), b0)
+    cx, _, _ = buf.combine(y, handle, bias=(b0.to(DEV), b1.to(DEV)))
+    assert torch.equal(cx.cpu(), (b0.float() + b1.float()).to(torch.bfloat16))
+    buf.destroy()
+
+
+@pytest.mark.parametrize('T,maxT,H,E,K,A,masked,fused', [
+    (33, 64, 384, 6, 1, 1, 0.0, False),        # top-1, hidden not a multiple of 512
+    (100, 100, 1040, 10, 3, 3, 0.2, True),     # odd top-k (generic combine), odd alignment, ragged last group
+    (257, 300, 2064, 40, 5, 16, 0.3, True),
+    (129, 129, 7168, 256, 7, 128, 0.0, False),
+    (5, 4096, 512, 64, 8, 64, 0.0, True),      # far fewer tokens than the buffer allows
+    (1000, 1000, 128, 4, 4, 32, 0.0, False),   # every token on every expert
+])
+def test_ragged_shapes(T, maxT, H, E, K, A, masked, fused):
+    x = make_tokens(T, H, seed=T, outliers=True)
+    topk, w = make_routing(T, E, K, seed=T, masked=masked)
+    _roundtrip(T, maxT, H, E, K, A, topk, w, x, fused=fused, seed=T)
+
+
+def test_duplicate_experts_in_a_row_are_legal():
+    T, H, E, K = 50, 256, 4, 4
+    x = make_tokens(T, H)
+    topk, w = make_routing(T, E, K, seed=1)
+    topk[:, 1] = topk[:, 0]
+    topk[::3, 3] = topk[::3, 2]
+    _roundtrip(T, T, H, E, K, 4, topk, w, x)
+    _roundtrip(T, T, H, E, K, 4, topk, w, x, R=2, rank=1)
+
+
+def test_current_stream_and_input_lifetime():
+    """Everything runs on the caller's current stream; inputs released right after the call stay valid
+    for the deferred epilogue even when the allocator hands their memory to someone else."""
+    import deep_ep
+    T, H, E = 16, 1024, 4
+    buf = _buffer(T, H, 1)
+    stream = torch.cuda.Stream()
+    for defer in (False, True):
+        for it in range(2):
+            with torch.cuda.stream(stream):
+                x = torch.empty((T, H), dtype=torch.bfloat16, device=DEV)
+                topk = torch.full((T, 1), it % E, dtype=torch.int64, device=DEV)
+                if it:
+                    torch.cuda._sleep(50_000_000)
+                x.fill_(1 + 10 * it)
+                res = buf.dispatch(x, topk_idx=topk, num_experts=E, expert_alignment=1, do_cpu_sync=False,
+                                   do_expand=True, async_with_compute_stream=True, defer_epilogue=defer)
+                assert torch.cuda.current_stream() == stream
+                if defer:
+                    ev = res
+                else:
+                    rx, _, _, handle, ev = res
+                    snap = rx[:T].clone()
+            del x
+            with torch.cuda.stream(stream):
+                pressure = torch.full((T, H), -100, dtype=torch.bfloat16, device=DEV)
+                if defer:
+                    rx, _, _, handle = ev.wait()
+                    snap = rx[:T].clone()
+                else:
+                    ev.wait()
+            stream.synchronize()
+            assert int(handle.psum_num_recv_tokens_per_rank[-1]) == T
+            assert torch.equal(snap, torch.full_like(snap, 1 + 10 * it))
+            del pressure
+    # events: a hook registered on an EventOverlap runs once, on the waiting stream
+    producer, consumer = torch.cuda.Stream(), torch.cuda.Stream()
+    src = torch.zeros(4096, device=DEV)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(producer):
+        torch.cuda._sleep(50_000_000)
+        src.fill_(3)
+        ready = deep_ep.EventHandle()
+    with torch.cuda.stream(stream):
+        ready.current_stream_wait()
+        mid = src * 2
+        ev = deep_ep.EventOverlap(deep_ep.EventHandle())
+    calls = []
+    ev.register_hook_after_wait(lambda: calls.append(torch.cuda.current_stream()) or mid + 1)
+    with torch.cuda.stream(consumer):
+        out = ev.wait()
+        assert ev.wait() is None
+    consumer.synchronize()
+    assert calls == [consumer] and torch.equal(out, torch.full_like(out, 7))
+    buf.destroy()
+
+
+def test_running_expert_statistics_accumulate():
+    T, H, E, K = 120, 256, 16, 4
+    x = make_tokens(T, H).to(DEV)
+    stats = torch.zeros(E, dtype=torch.int32, device=DEV)
+    buf = _buffer(T, H, K)
+    total = np.zeros(E, dtype=np.int64)
+    for seed in range(3):
+        topk, _ = make_routing(T, E, K, seed=seed, masked=0.1)
+        buf.dispatch(x, topk_idx=topk.to(DEV), cumulative_local_expert_recv_stats=stats, num_experts=E,
+                     do_expand=True)
+        total += np.bincount(topk[topk >= 0].numpy(), minlength=E)
+    torch.cuda.synchronize()
+    assert np.array_equal(stats.cpu().numpy(), total)
+    buf.destroy()
+
+
+def test_handle_guards_topk_idx_against_mutation():
+    T, H, E, K = 32, 256, 8, 2
+    topk, w = make_routing(T, E, K)
+    tg = topk.to(DEV)
+    buf = _buffer(T, H, K)
+    rx, _, _, handle, _ = buf.dispatch(make_tokens(T, H).to(DEV), topk_idx=tg, num_experts=E, do_expand=True)
+    assert handle.topk_idx is tg
+    tg[0, 0] = 1
+    with pytest.raises(AssertionError, match='must not be modified'):
+        buf.combine(rx, handle)
+    buf.destroy()
+
+
+def test_deterministic_flag_gives_the_same_layout():
+    T, H, E, K, A = 300, 512, 32, 4, 16
+    x = make_tokens(T, H).to(DEV)
+    topk, w = make_routing(T, E, K, seed=9, masked=0.1)
+    outs = []
+    for det in (False, True):
+        import deep_ep
+        buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K,
+                               deterministic=det, explicitly_destroy=True)
+        rx, _, rw, h, ev = buf.dispatch(x, topk_idx=topk.to(DEV), topk_weights=w.to(DEV), num_experts=E,
+                                        expert_alignment=A, do_expand=True, do_zero_padding=True,
+                                        async_with_compute_stream=det)
+        if det:
+            ev.current_stream_wait()      # the canonicalising hook runs when the event is waited on
+        torch.cuda.synchronize()
+        outs.append((rx.clone(), rw.clone(), h.recv_src_metadata.clone()))
+        if det:
+            assert h.cached_recv_src_metadata_before_sort is not None
+        buf.destroy()
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    # inside every expert the valid rows ascend with the source token (the reference's sorted order)
+    meta = outs[0][2].cpu().numpy()
+    for e in range(E):
+        tt, jj = np.nonzero(topk.numpy()[meta[:, K]] == e)
+        assert np.all(np.diff(meta[tt, jj]) > 0)
