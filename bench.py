@@ -35,6 +35,8 @@ WORKLOADS = {
     'c3_headline': (16384, 7168, 256, 6, 128, True),
     'c2_bf16_top8': (4096, 7168, 256, 8, 128, False),
     'c1_small': (128, 256, 8, 2, 1, False),
+    'c4_decode_zipf': (128, 7168, 256, 8, 128, True),
+    'c5_ep32_share': (16384, 7168, 256, 6, 128, True),     # 32 partitions of 8 experts, this GPU = partition 5
 }
 
 
@@ -90,6 +92,74 @@ def cpu_baseline(H, E, K, A, fp8, sample_tokens):
                       f'(numpy/torch-CPU oracle, os.cpu_count()={os.cpu_count()})'}
 
 
+def timed_us(fn, n):
+    """Average duration of fn in microseconds, from events on the current stream (the launch stream)."""
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    v = [a.elapsed_time(b) * 1e3 for a, b in evs]
+    return sum(v) / len(v)
+
+
+def bench_partitioned(args, T, H, E, K, A, R=32, rank=5):
+    """One GPU's share of EP-R: pack into R partition-major regions + expand the own region, then the
+    owner-side partial reduce + the token-side final reduce over a combine buffer whose other partials are
+    synthetic.  Not the headline line: printed for the record when asked for."""
+    import deep_ep
+    dev = torch.device('cuda', 0)
+    x, topk, w = make_inputs(T, H, E, K)
+    xg, tg, wg = x.to(dev), topk.to(dev), w.to(dev)
+    buf = deep_ep.EPBuffer(deep_ep.LocalGroup(rank, R), num_max_tokens_per_rank=T, hidden=H, num_topk=K,
+                           use_fp8_dispatch=True, explicitly_destroy=True)
+    kw = dict(num_experts=E, num_max_tokens_per_rank=T, expert_alignment=A, do_expand=True, do_zero_padding=True,
+              fused_fp8_quant=True)
+    (rx, rsf), _, rw, handle, _ = buf.dispatch(xg, topk_idx=tg, topk_weights=wg, **kw)
+    y = torch.randn((rx.size(0), H), device=dev).to(torch.bfloat16)
+    arena = buf.runtime.buffer_tensor()
+    ctok = H * 2 + -(-4 * K // 32) * 32
+    arena[:min(K, R) * T * ctok].view(torch.int16).random_(0, 0x3f80)       # finite BF16 partials everywhere
+    torch.cuda.synchronize()
+    n_send = int((handle.dst_buffer_slot_idx >= 0).sum())
+    n_recv = int(handle.psum_num_recv_tokens_per_rank[-1])
+    n_valid = int(handle.num_unaligned_recv_tokens_per_expert.sum())
+    tok = H + 224 + 96
+    b_pack = T * H * 2 + T * K * 12 + n_send * tok
+    b_expand = n_recv * tok + n_valid * (H + 224 + 4) + n_recv * (K + 2) * 4
+    b_partial = n_valid * H * 2 + n_recv * ctok + n_recv * (K + 2) * 4
+    b_final = n_send * ctok + T * H * 2 + T * K * 8 + T * K * 4
+
+    def step():
+        _, _, rw2, h, _ = buf.dispatch(xg, topk_idx=tg, topk_weights=wg, **kw)
+        buf.combine(y, h, topk_weights=rw2)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    us_d = timed_us(lambda: buf.dispatch(xg, topk_idx=tg, topk_weights=wg, **kw), args.steps)
+    us_c = timed_us(lambda: buf.combine(y, handle, topk_weights=rw), args.steps)
+    out = {'metric': 'dispatch & combine GB/s, one GPU share of EP32 (pack 32 regions + expand own; partial + final reduce)',
+           'value': round((b_pack + b_expand + b_partial + b_final) / ms / 1e6, 1), 'unit': 'GB/s', 'n_gpus': 1,
+           'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms, 4), 'higher_is_better': True,
+           'scaling': 'weak', 'vs_baseline': None, 'dtype': 'fp8_e4m3+bf16 payload, fp32 accumulate', 'data': 'synthetic',
+           'config': {'workload': args.workload, 'tokens': T, 'hidden': H, 'experts': E, 'topk': K,
+                      'expert_alignment': A, 'partitions': R, 'partition_idx': rank, 'packed_rows': n_send,
+                      'received_rows': n_recv, 'valid_expanded_rows': n_valid},
+           'phases': {'dispatch_us': round(us_d, 2), 'dispatch_bytes': b_pack + b_expand,
+                      'dispatch_gbs': round((b_pack + b_expand) / us_d / 1e3, 1),
+                      'combine_us': round(us_c, 2), 'combine_bytes': b_partial + b_final,
+                      'combine_gbs': round((b_partial + b_final) / us_c / 1e3, 1)}}
+    buf.destroy()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -118,6 +188,9 @@ def main():
             dst.copy_(src)          # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
+    if args.workload == 'c5_ep32_share':
+        bench_partitioned(args, T, H, E, K, A)
+        return
     x, topk, w = make_inputs(T, H, E, K)
     xg, tg, wg = x.to(dev), topk.to(dev), w.to(dev)
     buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K,
