@@ -24,8 +24,10 @@ _lib = ctypes.CDLL(_LIB_PATH)
 
 
 class _Tensor(ctypes.Structure):
+    # ep_tensor_t; size[2] and stride[2] are spelled out so one positional constructor call fills it
     _fields_ = [('data', ctypes.c_void_p), ('dtype', ctypes.c_int32), ('ndim', ctypes.c_int32),
-                ('size', ctypes.c_int64 * 2), ('stride', ctypes.c_int64 * 2)]
+                ('size0', ctypes.c_int64), ('size1', ctypes.c_int64),
+                ('stride0', ctypes.c_int64), ('stride1', ctypes.c_int64)]
 
 
 class _DispatchArgs(ctypes.Structure):
@@ -103,23 +105,21 @@ _DTYPES = {torch.bfloat16: 1, torch.float8_e4m3fn: 2, torch.int16: 3, torch.int3
            torch.float32: 6, torch.uint8: 7}
 
 
+_ABSENT = _Tensor()
+
+
 def _desc(t: Optional[torch.Tensor], two_byte_packs: bool = False) -> _Tensor:
-    d = _Tensor()
     if t is None:
-        return d
+        return _ABSENT
     if not t.is_cuda:
         raise EPException('every tensor handed to the EP kernels must live on the GPU')
-    assert 1 <= t.dim() <= 2
-    d.data = t.data_ptr() if t.numel() > 0 else _nonnull_ptr(t)
-    if two_byte_packs and t.element_size() == 2:
-        d.dtype = 3
-    else:
-        d.dtype = _DTYPES.get(t.dtype, 0)
-    d.ndim = t.dim()
-    for i in range(t.dim()):
-        d.size[i] = t.size(i)
-        d.stride[i] = t.stride(i)
-    return d
+    dtype = 3 if (two_byte_packs and t.element_size() == 2) else _DTYPES.get(t.dtype, 0)
+    ptr = t.data_ptr() or _nonnull_ptr(t)
+    shape, stride = t.shape, t.stride()
+    if len(shape) == 2:
+        return _Tensor(ptr, dtype, 2, shape[0], shape[1], stride[0], stride[1])
+    assert len(shape) == 1
+    return _Tensor(ptr, dtype, 1, shape[0], 0, stride[0], 0)
 
 
 _dummy = {}
@@ -134,7 +134,8 @@ def _nonnull_ptr(t: torch.Tensor) -> int:
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    # raw hipStream_t of the current stream of the current device
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
 
 # ---- module-level API -------------------------------------------------------------------------
@@ -383,8 +384,11 @@ class EPBuffer(BufferBase):
         a.stream = _stream()
         _check(_ep_dispatch(self._h, ctypes.byref(a)))
 
+        keep_alive = (x, sf, topk_idx, topk_weights, psum_rank, psum_expert)
+
         def epilogue():
-            # the inputs stay referenced by this closure until the copy kernel has been enqueued
+            # the descriptors hold raw pointers: the inputs stay referenced until the copy kernel is enqueued
+            assert keep_alive is not None
             per_expert_list: List[int] = []
             if cached_mode:
                 num_recv, num_expanded = cached_num_recv_tokens, cached_num_expanded_tokens
@@ -423,8 +427,9 @@ class EPBuffer(BufferBase):
                 recv_src_metadata = ints(alloc_recv, num_topk + 2)
 
             e = _DispatchEpilogueArgs()
-            e.x, e.sf, e.topk_weights = _desc(x), _desc(sf, two_byte_packs=True), _desc(topk_weights)
-            e.psum_num_recv_tokens_per_rank, e.psum_num_recv_tokens_per_expert = _desc(psum_rank), _desc(psum_expert)
+            e.x, e.sf, e.topk_weights = a.x, a.sf, a.topk_weights
+            e.psum_num_recv_tokens_per_rank = a.psum_num_recv_tokens_per_rank
+            e.psum_num_recv_tokens_per_expert = a.psum_num_recv_tokens_per_expert
             e.recv_x, e.recv_sf = _desc(recv_x), _desc(recv_sf, two_byte_packs=not fused_fp8_quant)
             e.recv_topk_weights, e.recv_src_metadata = _desc(recv_topk_weights), _desc(recv_src_metadata)
             e.num_topk, e.num_max_tokens_per_rank = num_topk, num_max_tokens_per_rank
@@ -473,28 +478,28 @@ class EPBuffer(BufferBase):
         hidden = x.size(1)
         num_combined_tokens, num_topk = combined_topk_idx.shape
 
-        def fill(combined_x, combined_topk_weights) -> _CombineArgs:
-            c = _CombineArgs()
-            c.x, c.topk_weights, c.bias_0, c.bias_1 = _desc(x), _desc(topk_weights), _desc(bias_0), _desc(bias_1)
-            c.src_metadata, c.combined_topk_idx = _desc(src_metadata), _desc(combined_topk_idx)
-            c.psum_num_recv_tokens_per_rank = _desc(psum_num_recv_tokens_per_rank)
-            c.combined_x, c.combined_topk_weights = _desc(combined_x), _desc(combined_topk_weights)
-            c.num_experts, c.num_max_tokens_per_rank = num_experts, num_max_tokens_per_rank
-            c.apply_weights = int(apply_weights)
-            c.stream = _stream()
-            return c
+        c = _CombineArgs()
+        c.x, c.topk_weights, c.bias_0, c.bias_1 = _desc(x), _desc(topk_weights), _desc(bias_0), _desc(bias_1)
+        c.src_metadata, c.combined_topk_idx = _desc(src_metadata), _desc(combined_topk_idx)
+        c.psum_num_recv_tokens_per_rank = _desc(psum_num_recv_tokens_per_rank)
+        c.num_experts, c.num_max_tokens_per_rank = num_experts, num_max_tokens_per_rank
+        c.apply_weights = int(apply_weights)
+        c.stream = _stream()
+        _check(_ep_combine(self._h, ctypes.byref(c), 0))           # owner side (nothing to do for one partition)
 
-        c0 = fill(None, None)
-        _check(_ep_combine(self._h, ctypes.byref(c0), 0))
+        keep_alive = (x, topk_weights, bias_0, bias_1, src_metadata, combined_topk_idx, psum_num_recv_tokens_per_rank)
 
         def epilogue():
+            # the descriptors hold raw pointers: the tensors stay referenced until the reduce is enqueued
+            assert keep_alive is not None
             combined_x = torch.empty((num_combined_tokens, hidden), dtype=x.dtype, device=dev)
             combined_topk_weights = None
             if topk_weights is not None:
                 combined_topk_weights = torch.empty((num_combined_tokens, num_topk), dtype=topk_weights.dtype,
                                                     device=dev)
-            c1 = fill(combined_x, combined_topk_weights)
-            _check(_ep_combine(self._h, ctypes.byref(c1), 1))
+            c.combined_x, c.combined_topk_weights = _desc(combined_x), _desc(combined_topk_weights)
+            c.stream = _stream()
+            _check(_ep_combine(self._h, ctypes.byref(c), 1))       # token side
             return combined_x, combined_topk_weights
 
         if defer_epilogue:
