@@ -14,6 +14,9 @@
 #define EP_ROWS_PER_BLOCK 4
 #define EP_PAD_BLOCKS_PER_EXPERT 4
 
+#define EP_LAYOUT_SCANNED 0
+#define EP_LAYOUT_SINGLE 2
+
 #define EP_SCATTER_EXPAND 0
 #define EP_SCATTER_PACK 1
 #define EP_SCATTER_REGION 2
@@ -38,7 +41,7 @@ struct EpLayoutArgs {
     int num_blocks;               // ceil(T / EP_TOKENS_PER_BLOCK), at least 1
     int seq;                      // value the host waits for in host_page[0]
     int notify_host;              // do_cpu_sync
-    int pad0;
+    int scan_mode;                // EP_LAYOUT_*: where ep_layout_assign finds the other blocks' counts
     // scratch (device)
     int* blk_expert_cnt;          // [num_blocks, E]   counts, then exclusive prefix over blocks
     int* blk_rank_cnt;            // [num_blocks, R]   master counts, then exclusive prefix

@@ -151,29 +151,80 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
 //                               with the canonical order of deep_ep/buffers/ep.py:100-160
 // Block 0 also publishes the per-partition / per-expert counts and prefix sums
 // (impls/ep/dispatch.hpp:469-545) and, when asked, the host count page.
+//
+// Where the counts of the other blocks come from (a.scan_mode):
+//   EP_LAYOUT_SCANNED  ep_layout_scan left exclusive prefixes in blk_*_cnt and totals in *_total
+//   EP_LAYOUT_SINGLE   one block owns every token: nothing ran before, its own LDS counts are the totals
+// Only the local experts and the partitions need prefixes: slots of other experts are never used.
 // ------------------------------------------------------------------------------------------------
+#define EP_LAYOUT_MAX_COLS_PER_THREAD ((EP_MAX_EXPERTS + EP_MAX_RANKS + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS)
+
 extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign(EpLayoutArgs a) {
     extern __shared__ int smem[];
     const int E = a.num_experts, R = a.num_ranks, K = a.num_topk, El = a.experts_per_rank, A = a.expert_alignment;
     const int NW = EP_LAYOUT_THREADS / WAVE;
-    int* s_start = smem;                   // [El] first slot of each local expert
-    int* s_we = s_start + El;              // [NW][E] running slot counters per wave
+    const int b = blockIdx.x;
+    int* s_tot = smem;                     // [El + R] totals of the local experts, then of the partitions
+    int* s_we = s_tot + El + R;            // [NW][E] per-wave counts, then running slot counters
     int* s_wr = s_we + NW * E;             // [NW][R]
     int* s_tmp = s_wr + NW * R;            // [NW + 1]
     short* s_key = (short*)(s_tmp + NW + 1);
     short* s_rk = s_key + EP_TOKENS_PER_BLOCK * K;
     const int tid = threadIdx.x, lane = lane_id(), w = wave_id();
     const int lo = a.rank_idx * El;
+    const int ncols = El + R;              // column c < El: local expert lo + c; else partition c - El
 
-    // ---- aligned exclusive scan over the local experts (every block recomputes it: El <= 2048) ----
-    const int per = (El + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS;
-    const int e0 = tid * per, e1 = min(El, e0 + per);
-    int mine = 0;
-    for (int e = e0; e < e1; ++e) mine += align_up(a.expert_total[lo + e], A);
-    const int incl = wave_inclusive_sum(mine);
-    if (lane == WAVE - 1) s_tmp[w] = incl;
+    // ---- A: stage this block's keys, clear the per-wave counters ----
     for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
     layout_load_keys(a, s_key, s_rk);
+    __syncthreads();
+
+    // ---- B: per-wave counts: wave w owns entries [w*epw, (w+1)*epw) of this block's chunk ----
+    const int n = EP_TOKENS_PER_BLOCK * K;
+    const int rounds = (n + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS;
+    const int epw = rounds * WAVE;
+    for (int rd = 0; rd < rounds; ++rd) {
+        const int idx = w * epw + rd * WAVE + lane;
+        if (idx < n) {
+            const int e = s_key[idx];
+            if (e >= 0) atomicAdd(&s_we[w * E + e], 1);
+            const int mr = master_rank(s_rk, idx, K);
+            if (mr >= 0) atomicAdd(&s_wr[w * R + mr], 1);
+        }
+    }
+    __syncthreads();
+
+    // ---- C: counts of the blocks before this one (kept in registers) and totals over all blocks ----
+    int pre[EP_LAYOUT_MAX_COLS_PER_THREAD];
+#pragma unroll
+    for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
+        pre[k] = 0;
+        const int c = tid + k * EP_LAYOUT_THREADS;
+        if (c >= ncols) continue;
+        const bool is_expert = c < El;
+        const int col = is_expert ? lo + c : c - El;
+        const int stride = is_expert ? E : R;
+        int tot = 0;
+        if (a.scan_mode == EP_LAYOUT_SCANNED) {
+            pre[k] = (is_expert ? a.blk_expert_cnt : a.blk_rank_cnt)[(int64_t)b * stride + col];
+            tot = is_expert ? a.expert_total[col] : a.rank_total[col];
+        } else {
+            const int* wc = is_expert ? s_we + col : s_wr + col;
+            for (int i = 0; i < NW; ++i) tot += wc[i * stride];
+        }
+        s_tot[c] = tot;
+    }
+    __syncthreads();
+
+    // ---- D + E: aligned exclusive scan over the local experts (totals are replaced in place by the
+    //      first slot of each expert); block 0 publishes the handle tensors and the host count page ----
+    int* s_start = s_tot;
+    const int per = (El + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS;
+    const int e0 = min(El, tid * per), e1 = min(El, e0 + per);
+    int mine = 0;
+    for (int e = e0; e < e1; ++e) mine += align_up(s_tot[e], A);
+    const int incl = wave_inclusive_sum(mine);
+    if (lane == WAVE - 1) s_tmp[w] = incl;
     __syncthreads();
     int wave_off = 0, grand = 0;
     for (int i = 0; i < NW; ++i) {
@@ -183,21 +234,19 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     {
         int run = wave_off + incl - mine;
         for (int e = e0; e < e1; ++e) {
+            const int c = s_tot[e];
+            if (b == 0) {
+                a.unaligned_expert[e] = c;
+                a.psum_expert[e] = run + c;
+                if (a.cumulative_stats != nullptr) atomicAdd(&a.cumulative_stats[e], c);
+                if (a.notify_host) a.host_page[EP_HOST_EXPERT_OFF + e] = align_up(c, A);
+            }
             s_start[e] = run;
-            run += align_up(a.expert_total[lo + e], A);
+            run += align_up(c, A);
         }
     }
-    __syncthreads();
-
-    if (blockIdx.x == 0) {
-        const int n_self = a.rank_total[a.rank_idx];
-        for (int e = tid; e < El; e += blockDim.x) {
-            const int c = a.expert_total[lo + e];
-            a.unaligned_expert[e] = c;
-            a.psum_expert[e] = s_start[e] + c;
-            if (a.cumulative_stats != nullptr) atomicAdd(&a.cumulative_stats[e], c);
-            if (a.notify_host) a.host_page[EP_HOST_EXPERT_OFF + e] = align_up(c, A);
-        }
+    if (b == 0) {
+        const int n_self = s_tot[El + a.rank_idx];
         for (int r = tid; r < R; r += blockDim.x) {
             a.psum_rank[r] = r >= a.rank_idx ? n_self : 0;
             if (a.notify_host) a.host_page[EP_HOST_RANK_OFF + r] = r == a.rank_idx ? n_self : 0;
@@ -213,42 +262,26 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             }
         }
     }
-
-    // ---- per-wave counts: wave w owns entries [w*epw, (w+1)*epw) of this block's chunk ----
-    const int n = EP_TOKENS_PER_BLOCK * K;
-    const int rounds = (n + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS;
-    const int epw = rounds * WAVE;
-    for (int rd = 0; rd < rounds; ++rd) {
-        const int idx = w * epw + rd * WAVE + lane;
-        if (idx < n) {
-            const int e = s_key[idx];
-            if (e >= 0) atomicAdd(&s_we[w * E + e], 1);
-            const int mr = master_rank(s_rk, idx, K);
-            if (mr >= 0) atomicAdd(&s_wr[w * R + mr], 1);
-        }
-    }
     __syncthreads();
-    // counts -> starting slots (global base + blocks before + waves before)
-    for (int e = tid; e < E; e += blockDim.x) {
-        const int le = e - lo;
-        int run = a.blk_expert_cnt[(int64_t)blockIdx.x * E + e] + ((le >= 0 && le < El) ? s_start[le] : 0);
+
+    // ---- F: counts -> starting slots (global base + blocks before + waves before) ----
+#pragma unroll
+    for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
+        const int c = tid + k * EP_LAYOUT_THREADS;
+        if (c >= ncols) continue;
+        const bool is_expert = c < El;
+        int* wc = is_expert ? s_we + lo + c : s_wr + (c - El);
+        const int stride = is_expert ? E : R;
+        int run = pre[k] + (is_expert ? s_start[c] : 0);
         for (int i = 0; i < NW; ++i) {
-            const int c = s_we[i * E + e];
-            s_we[i * E + e] = run;
-            run += c;
-        }
-    }
-    for (int r = tid; r < R; r += blockDim.x) {
-        int run = a.blk_rank_cnt[(int64_t)blockIdx.x * R + r];
-        for (int i = 0; i < NW; ++i) {
-            const int c = s_wr[i * R + r];
-            s_wr[i * R + r] = run;
-            run += c;
+            const int cnt = wc[i * stride];
+            wc[i * stride] = run;
+            run += cnt;
         }
     }
     __syncthreads();
 
-    // ---- stable ranking, 64 consecutive entries per wave per round ----
+    // ---- G: stable ranking, 64 consecutive entries per wave per round ----
     const int ebits = 32 - __builtin_clz(E);       // keys+1 in [0, E]
     const int rbits = 32 - __builtin_clz(R);
     const uint64_t lt = (1ull << lane) - 1ull;
@@ -257,11 +290,13 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
         const int idx = w * epw + rd * WAVE + lane;
         const bool in = idx < n;
         const int e = in ? s_key[idx] : -1;
+        const int le = e - lo;
+        const bool local = e >= 0 && le >= 0 && le < El;
         const int mr = in ? master_rank(s_rk, idx, K) : -1;
-        const uint64_t pe = match_any(e + 1, ebits);
+        const uint64_t pe = match_any(local ? e + 1 : 0, ebits);
         const uint64_t pr = match_any(mr + 1, rbits);
         int eslot = -1, rslot = -1;
-        if (e >= 0) {
+        if (local) {
             eslot = s_we[w * E + e] + __popcll(pe & lt);
             if ((pe >> lane) == 1ull) s_we[w * E + e] = eslot + 1;      // highest peer advances the counter
         }
@@ -269,15 +304,16 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             rslot = s_wr[w * R + mr] + __popcll(pr & lt);
             if ((pr >> lane) == 1ull) s_wr[w * R + mr] = rslot + 1;
         }
-        const int64_t g = (int64_t)blockIdx.x * n + idx;
+        const int64_t g = (int64_t)b * n + idx;
         if (in && g < total) {
-            const int le = e - lo;
             a.dst_buffer_slot_idx[g] = rslot;
             a.dst_gsge_idx[g] = -1;                 // every copy is local: no transport descriptors
-            a.slot_map[g] = (e >= 0 && le >= 0 && le < El) ? eslot : -1;
-            if (mr == a.rank_idx && rslot < a.max_tokens) a.recv_tok[rslot] = (int)(g / K);
+            a.slot_map[g] = eslot;
+            if (mr == a.rank_idx && rslot < a.max_tokens) a.recv_tok[rslot] = b * EP_TOKENS_PER_BLOCK + idx / K;
         }
-        __syncthreads();
+        // the running counters of a wave are touched by that wave only and the LDS operations of a wave
+        // complete in order: no block barrier (which would also wait for the stores above) is needed
+        __builtin_amdgcn_wave_barrier();
     }
 }
 

@@ -534,10 +534,14 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         const unsigned smem_count = (unsigned)(E + R) * sizeof(int) + key_bytes;
         const unsigned nw = EP_LAYOUT_THREADS / 64;
         const unsigned smem_assign =
-            (unsigned)(num_experts_per_rank + nw * (E + R) + nw + 1) * sizeof(int) + key_bytes;
+            (unsigned)(num_experts_per_rank + R + nw * (E + R) + nw + 1) * sizeof(int) + key_bytes;
         EP_HOST_ASSERT(smem_assign <= 64 * 1024);
-        launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, smem_count, a.stream, la);
-        launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 64), EP_SCAN_THREADS, 0, a.stream, la);
+        // one block: its own counts are the totals and nothing has to run before the slot assignment
+        la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : EP_LAYOUT_SCANNED;
+        if (la.scan_mode != EP_LAYOUT_SINGLE)
+            launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, smem_count, a.stream, la);
+        if (la.scan_mode == EP_LAYOUT_SCANNED)
+            launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 64), EP_SCAN_THREADS, 0, a.stream, la);
         launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, a.stream, la);
 
         if (num_ranks > 1) launch_pack();

@@ -18,7 +18,7 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'lib')
 _LIB_PATH = os.path.join(_LIB_DIR, 'libdeep_ep_hip.so')
 
 if not os.path.exists(_LIB_PATH):
-    raise ImportError(f'{_LIB_PATH} is missing: build the native library first (python -m deep_ep._build)')
+    raise ImportError(f'{_LIB_PATH} is missing: build the native library first (python deepep-ascend_amd/deep_ep/_build.py)')
 
 _lib = ctypes.CDLL(_LIB_PATH)
 

@@ -3,7 +3,7 @@
   deep_ep/lib/ep_kernels.hsaco     device code object   (hipcc --genco)
   deep_ep/lib/libdeep_ep_hip.so    host runtime, C ABI  (hipcc -shared)
 
-hipcc cross-compiles, so this runs on a machine without a GPU.  `python -m deep_ep._build`.
+hipcc cross-compiles, so this runs on a machine without a GPU.  `python deepep-ascend_amd/deep_ep/_build.py`.
 """
 import os
 import subprocess

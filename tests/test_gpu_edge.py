@@ -215,3 +215,21 @@ def test_deterministic_flag_gives_the_same_layout():
     for e in range(E):
         tt, jj = np.nonzero(topk.numpy()[meta[:, K]] == e)
         assert np.all(np.diff(meta[tt, jj]) > 0)
+
+
+@pytest.mark.parametrize('T,E,K,R,rank', [(700, 64, 6, 1, 0), (1500, 256, 8, 8, 3), (300, 2048, 4, 1, 0), (128, 256, 8, 1, 0),
+                                         (129, 256, 8, 4, 2)])
+def test_single_and_multi_block_layouts_agree_with_oracle(T, E, K, R, rank):
+    """128 tokens fit one layout block (no counting pass runs); 129 need the counting and scan passes."""
+    H, A = 128, 16
+    topk, w = make_routing(T, E, K, seed=T, masked=0.1)
+    lay = O.rank_share_layout(topk.numpy(), E, R, rank, A, T)
+    buf = _buffer(T, H, K, R, rank)
+    _, _, _, handle, _ = buf.dispatch(make_tokens(T, H).to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV),
+                                      num_experts=E, expert_alignment=A, do_expand=True)
+    torch.cuda.synchronize()
+    for name in ('psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
+                 'num_unaligned_recv_tokens_per_expert', 'dst_buffer_slot_idx', 'recv_src_metadata'):
+        assert np.array_equal(getattr(handle, name).cpu().numpy(), lay[name]), name
+    assert handle.num_recv_tokens_per_expert_list == lay['num_recv_tokens_per_expert_list']
+    buf.destroy()
