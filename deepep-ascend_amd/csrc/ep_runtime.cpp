@@ -210,6 +210,18 @@ struct ep_buffer {
     char* lb() const { return arena + kWorkspaceBytes + num_buffer_bytes; }
 };
 
+namespace {
+// The code object is loaded on one device and the arena lives there: calls must come with that
+// device current.
+void check_buffer(const ep_buffer* b) {
+    EP_HOST_ASSERT(b != nullptr);
+    EP_HOST_ASSERT(not b->destroyed);
+    int dev = -1;
+    HIP_CHECK(hipGetDevice(&dev));
+    EP_HOST_ASSERT(dev == b->device and "the buffer belongs to another device");
+}
+}  // namespace
+
 extern "C" {
 
 const char* ep_last_error(void) { return g_err.c_str(); }
@@ -291,6 +303,9 @@ int ep_buffer_create(int rank_idx, int num_ranks, int64_t num_bytes, int64_t num
         EP_HOST_ASSERT(num_ranks > 0 and num_ranks <= EP_MAX_RANKS and rank_idx >= 0 and rank_idx < num_ranks);
         EP_HOST_ASSERT(cpu_timeout_secs > 0 and gpu_timeout_secs > 0);
         load_kernels(nullptr);
+        int cur = -1;
+        HIP_CHECK(hipGetDevice(&cur));
+        EP_HOST_ASSERT(cur == g_k.device and "the kernels were loaded on another device");
         auto* b = new ep_buffer();
         b->rank_idx = rank_idx;
         b->num_ranks = num_ranks;
@@ -356,8 +371,8 @@ int ep_buffer_print_memory_usage(ep_buffer_t* b) {
 // ---- dispatch ---------------------------------------------------------------------------------
 int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
     return guarded([&] {
-        EP_HOST_ASSERT(b != nullptr and pa != nullptr);
-        EP_HOST_ASSERT(not b->destroyed);
+        EP_HOST_ASSERT(pa != nullptr);
+        check_buffer(b);
         const ep_dispatch_args_t& a = *pa;
         const bool cached_mode = a.cached_mode != 0;
         const bool do_cpu_sync = a.do_cpu_sync != 0;
@@ -593,8 +608,8 @@ int ep_dispatch_worst_case_sizes(ep_buffer_t* b, int max_tokens, int num_topk, i
 
 int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_t* pa) {
     return guarded([&] {
-        EP_HOST_ASSERT(b != nullptr and pa != nullptr);
-        EP_HOST_ASSERT(not b->destroyed);
+        EP_HOST_ASSERT(pa != nullptr);
+        check_buffer(b);
         const ep_dispatch_epilogue_args_t& a = *pa;
         const bool cached_mode = a.cached_mode != 0;
         EP_HOST_ASSERT(present(a.x) and a.x.ndim == 2 and contiguous(a.x));
@@ -709,8 +724,8 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
 // ---- combine ----------------------------------------------------------------------------------
 int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
     return guarded([&] {
-        EP_HOST_ASSERT(b != nullptr and pa != nullptr);
-        EP_HOST_ASSERT(not b->destroyed);
+        EP_HOST_ASSERT(pa != nullptr);
+        check_buffer(b);
         const ep_combine_args_t& a = *pa;
         const int R = b->num_ranks;
         EP_HOST_ASSERT(a.num_experts > 0 and a.num_experts % R == 0);
