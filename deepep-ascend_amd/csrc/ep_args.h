@@ -59,6 +59,13 @@ struct EpLayoutArgs {
     int* host_page;               // device view of the mapped host page
 };
 
+// recv_sf layouts: rows of scales, or columns of scales whose stride is the row count of recv_sf
+// (EP_SF_COL_MAJOR) or the expanded row count the layout pass produced (EP_SF_COL_MAJOR_COUNTED:
+// the host does not know it yet when the kernel is enqueued).
+#define EP_SF_ROW_MAJOR 0
+#define EP_SF_COL_MAJOR 1
+#define EP_SF_COL_MAJOR_COUNTED 2
+
 // One receive-stream row per wave: copy (or quantise) it into every expanded slot it owns.
 struct EpScatterArgs {
     const void* x;                // [T, hidden] rows: BF16, or FP8 bytes when prequantised
@@ -96,6 +103,8 @@ struct EpScatterArgs {
     int with_metadata;            // packed rows carry topk_idx and the source token (non-cached)
     int idx_off, w_off, src_off;  // byte offsets of the packed metadata inside a row
     int num_out_rows;             // rows of recv_x: slots outside are ignored
+    int sf_col_major;             // EP_SF_* layout of recv_sf
+    int sf_elem_bytes;            // element size of recv_sf: 2 (packs) or 4 (fp32 scales)
     int pad0;
 };
 

@@ -474,6 +474,8 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             sa.copy_bytes = sa.x_row_bytes;
             sa.out_row_bytes = pk.bytes;
             sa.out_sf_row_bytes = pk.bytes;
+            sa.sf_col_major = EP_SF_ROW_MAJOR;
+            sa.sf_elem_bytes = a.fused_fp8_quant ? 4 : 2;
             if (present(a.sf)) {
                 sa.sf_token_stride_bytes = a.sf.stride[0] * 2;
                 sa.sf_pack_stride_bytes = a.sf.stride[1] * 2;
@@ -635,8 +637,13 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
                 EP_HOST_ASSERT(elem_size(a.recv_sf.dtype) == 2 and a.recv_sf.size[1] == a.sf.size[1]);
                 num_sf_packs = (int)a.sf.size[1];
             }
-            // the copy epilogue only writes row-major scale rows (csrc/kernels/ep/dispatch.hpp:112-113)
-            EP_HOST_ASSERT(a.recv_sf.stride[1] == 1 and a.recv_sf.stride[0] == a.recv_sf.size[1]);
+            // row-major scale rows (csrc/kernels/ep/dispatch.hpp:112-113), or the column-major result of
+            // the reference's transposing pass (csrc/buffers/ep.hpp:379-381) written in place
+            EP_HOST_ASSERT(a.recv_sf_layout >= EP_SF_ROW_MAJOR and a.recv_sf_layout <= EP_SF_COL_MAJOR_COUNTED);
+            if (a.recv_sf_layout == EP_SF_ROW_MAJOR)
+                EP_HOST_ASSERT(a.recv_sf.stride[1] == 1 and a.recv_sf.stride[0] == a.recv_sf.size[1]);
+            else
+                EP_HOST_ASSERT(a.recv_sf.stride[0] == 1 and a.recv_sf.stride[1] == a.recv_sf.size[0]);
         }
         if (present(a.topk_weights)) {
             EP_HOST_ASSERT(present(a.recv_topk_weights) and a.recv_topk_weights.ndim == 1);
@@ -666,6 +673,8 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.psum_expert = (const int*)a.psum_num_recv_tokens_per_expert.data;
         sa.out_row_bytes = (int64_t)hidden * elem_size(a.recv_x.dtype);
         sa.out_sf_row_bytes = has_sf ? a.recv_sf.size[1] * elem_size(a.recv_sf.dtype) : 0;
+        sa.sf_elem_bytes = has_sf ? elem_size(a.recv_sf.dtype) : 2;
+        sa.sf_col_major = has_sf ? a.recv_sf_layout : EP_SF_ROW_MAJOR;
         sa.hidden = hidden;
         sa.num_topk = K;
         // never walk past the rows the metadata tensor holds

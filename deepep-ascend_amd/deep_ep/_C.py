@@ -46,7 +46,7 @@ class _DispatchEpilogueArgs(ctypes.Structure):
         'recv_x', 'recv_sf', 'recv_topk_weights', 'recv_src_metadata')] + [
         ('num_topk', ctypes.c_int32), ('num_max_tokens_per_rank', ctypes.c_int32), ('num_experts', ctypes.c_int32),
         ('expert_alignment', ctypes.c_int32), ('cached_mode', ctypes.c_int32), ('do_zero_padding', ctypes.c_int32),
-        ('fused_fp8_quant', ctypes.c_int32), ('stream', ctypes.c_void_p)]
+        ('fused_fp8_quant', ctypes.c_int32), ('recv_sf_layout', ctypes.c_int32), ('stream', ctypes.c_void_p)]
 
 
 class _CombineArgs(ctypes.Structure):
@@ -412,10 +412,15 @@ class EPBuffer(BufferBase):
             out_dtype = torch.float8_e4m3fn if fused_fp8_quant else x.dtype
             recv_x = torch.empty((alloc_expanded, hidden), dtype=out_dtype, device=dev)
             recv_sf = None
-            if fused_fp8_quant:
-                recv_sf = torch.empty((alloc_expanded, (hidden + 127) // 128), dtype=torch.float32, device=dev)
-            elif sf is not None:
-                recv_sf = torch.empty((alloc_expanded, sf.size(1)), dtype=sf.dtype, device=dev)
+            if fused_fp8_quant or sf is not None:
+                sf_cols = (hidden + 127) // 128 if fused_fp8_quant else sf.size(1)
+                sf_dtype = torch.float32 if fused_fp8_quant else sf.dtype
+                if use_col_major_sf:
+                    # the copy kernel writes the scales column by column: no transposing pass afterwards
+                    sf_storage = torch.empty((sf_cols * alloc_expanded,), dtype=sf_dtype, device=dev)
+                    recv_sf = sf_storage.as_strided((alloc_expanded, sf_cols), (1, alloc_expanded))
+                else:
+                    recv_sf = torch.empty((alloc_expanded, sf_cols), dtype=sf_dtype, device=dev)
             recv_topk_weights = None
             if topk_weights is not None:
                 recv_topk_weights = torch.empty((alloc_expanded,), dtype=topk_weights.dtype, device=dev)
@@ -436,6 +441,8 @@ class EPBuffer(BufferBase):
             e.num_experts, e.expert_alignment = num_experts, expert_alignment
             e.cached_mode, e.do_zero_padding = int(cached_mode), int(do_zero_padding)
             e.fused_fp8_quant = int(fused_fp8_quant)
+            # sizes still unknown on the host: the column stride is the row count the device computed
+            e.recv_sf_layout = (2 if num_recv is None else 1) if use_col_major_sf else 0
             e.stream = _stream()
             _check(_ep_dispatch_epi(self._h, ctypes.byref(e)))
 
@@ -448,12 +455,13 @@ class EPBuffer(BufferBase):
                 if num_recv > alloc_recv or num_expanded > alloc_expanded:
                     raise EPException('Assertion exception (_C.py): received counts exceed this call\'s bound')
                 recv_x = recv_x[:num_expanded]
-                recv_sf = recv_sf[:num_expanded] if recv_sf is not None else None
+                if recv_sf is not None and use_col_major_sf:
+                    recv_sf = sf_storage.as_strided((num_expanded, sf_cols), (1, num_expanded))
+                elif recv_sf is not None:
+                    recv_sf = recv_sf[:num_expanded]
                 recv_topk_weights = recv_topk_weights[:num_expanded] if recv_topk_weights is not None else None
                 recv_src_metadata = recv_src_metadata[:num_recv]
 
-            if recv_sf is not None and use_col_major_sf:
-                recv_sf = recv_sf.transpose(0, 1).contiguous().transpose(0, 1)
             return (recv_x, recv_sf, recv_topk_weights, num_recv, num_expanded, per_expert_list,
                     psum_rank, psum_expert, unaligned, recv_src_metadata, dst_slot, dst_gsge)
 

@@ -165,6 +165,54 @@ def test_fp8_dispatch_fused_and_prequantised(T, H, E, K, A, masked, zipf):
     buf.destroy()
 
 
+@pytest.mark.parametrize('R,rank', [(1, 0), (4, 2)])
+@pytest.mark.parametrize('do_cpu_sync', [True, False])
+def test_column_major_scales_are_written_in_place(R, rank, do_cpu_sync):
+    """use_tma_aligned_col_major_sf: strides (1, N) exactly as the reference's transposing pass leaves
+    them (tests/ep/test_ep.py:141-145), for fused and pre-quantised input, with and without the host
+    sync, for a cached replay, and at R > 1 where fp32 scales travel as two 2-byte packs."""
+    de = _deep_ep()
+    T, H, E, K, A = 300, 1024, 16, 4, 32
+    x = make_tokens(T, H, seed=9, outliers=True)
+    topk, w = make_routing(T, E, K, seed=9, masked=0.2)
+    lay = O.rank_share_layout(topk.numpy(), E, R, rank, A, T)
+    q, s = O.quantise(x)
+    eq, es, ew = O.rank_share_dispatch(q.numpy(), s.numpy().view(np.uint32), w.numpy(), lay)
+    ne = lay['num_expanded_tokens']
+    buf = _buffer(T, H, K, R=R, rank=rank, fp8=True)
+    tg, wg = topk.to(DEV), w.to(DEV)
+    common = dict(num_experts=E, num_max_tokens_per_rank=T, expert_alignment=A, do_expand=True,
+                  do_zero_padding=True, do_cpu_sync=do_cpu_sync, use_tma_aligned_col_major_sf=True)
+
+    def check(rx, rsf, expect_q, expect_s, view):
+        n = rx.size(0)
+        assert n == (ne if do_cpu_sync else O.no_sync_sizes(R, T, K, E, A)[1])
+        assert rsf.shape == (n, expect_s.shape[1]) and rsf.stride() == (1, n)
+        assert np.array_equal(rx.view(torch.uint8).cpu().numpy()[:ne], expect_q)
+        assert np.array_equal(rsf.cpu().numpy().view(view)[:ne], expect_s)
+
+    (rx, rsf), _, rw, handle, _ = buf.dispatch(x.to(DEV), topk_idx=tg, topk_weights=wg, fused_fp8_quant=True, **common)
+    torch.cuda.synchronize()
+    check(rx, rsf, eq, es, np.uint32)
+
+    sf16 = s.view(torch.int16).to(DEV)
+    es16 = es.view(np.int16).reshape(ne, -1)
+    (px, psf), _, _, h2, _ = buf.dispatch((q.view(torch.float8_e4m3fn).to(DEV), sf16), topk_idx=tg, topk_weights=wg,
+                                          **common)
+    torch.cuda.synchronize()
+    check(px, psf, eq, es16, np.int16)
+
+    # cached replay with new payload
+    x2 = make_tokens(T, H, seed=10)
+    q2, s2 = O.quantise(x2)
+    eq2, es2, _ = O.rank_share_dispatch(q2.numpy(), s2.numpy().view(np.uint32), w.numpy(), lay)
+    (cx, csf), _, _, _, _ = buf.dispatch(x2.to(DEV), handle=handle, fused_fp8_quant=True, do_expand=True,
+                                         do_zero_padding=True, use_tma_aligned_col_major_sf=True)
+    torch.cuda.synchronize()
+    check(cx, csf, eq2, es2, np.uint32)
+    buf.destroy()
+
+
 def test_fp8_hardware_conversion_matches_integer_conversion():
     """Every fp32 bit pattern with |x| <= 464 (the quantiser never exceeds 448*(1+2^-23))."""
     de = _deep_ep()

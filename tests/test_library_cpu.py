@@ -129,3 +129,33 @@ def test_python_quantiser_matches_oracle(de):
     assert torch.equal(q.view(torch.uint8), oq) and torch.equal(s, os_)
     back = de.utils.math.per_token_cast_back(q, s)
     assert (back.float() - x.float()).abs().max() <= 0.07 * x.float().abs().max()
+
+
+def test_ctypes_structs_match_the_header(de, tmp_path):
+    """The Python binding restates the argument structs of the header: compile the header with gcc and
+    compare sizes and the offsets of the trailing fields."""
+    import subprocess
+    src = tmp_path / 'abi.c'
+    src.write_text('''
+#include <stdio.h>
+#include <stddef.h>
+#include "deep_ep_hip.h"
+int main(void) {
+    printf("%zu %zu %zu %zu\\n", sizeof(ep_tensor_t), sizeof(ep_dispatch_args_t),
+           sizeof(ep_dispatch_epilogue_args_t), sizeof(ep_combine_args_t));
+    printf("%zu %zu %zu %zu\\n", offsetof(ep_dispatch_args_t, stream), offsetof(ep_dispatch_args_t, fused_fp8_quant),
+           offsetof(ep_dispatch_epilogue_args_t, stream), offsetof(ep_dispatch_epilogue_args_t, recv_sf_layout));
+    printf("%zu %zu\\n", offsetof(ep_combine_args_t, stream), offsetof(ep_combine_args_t, apply_weights));
+    return 0;
+}
+''')
+    exe = tmp_path / 'abi'
+    subprocess.run(['gcc', '-I', os.path.join(ROOT, 'include'), '-o', str(exe), str(src)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    C = de._C
+    got = [ctypes.sizeof(C._Tensor), ctypes.sizeof(C._DispatchArgs), ctypes.sizeof(C._DispatchEpilogueArgs),
+           ctypes.sizeof(C._CombineArgs),
+           C._DispatchArgs.stream.offset, C._DispatchArgs.fused_fp8_quant.offset,
+           C._DispatchEpilogueArgs.stream.offset, C._DispatchEpilogueArgs.recv_sf_layout.offset,
+           C._CombineArgs.stream.offset, C._CombineArgs.apply_weights.offset]
+    assert got == [int(v) for v in out]
