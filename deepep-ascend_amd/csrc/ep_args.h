@@ -59,13 +59,6 @@ struct EpLayoutArgs {
     int* host_page;               // device view of the mapped host page
 };
 
-// recv_sf layouts: rows of scales, or columns of scales whose stride is the row count of recv_sf
-// (EP_SF_COL_MAJOR) or the expanded row count the layout pass produced (EP_SF_COL_MAJOR_COUNTED:
-// the host does not know it yet when the kernel is enqueued).
-#define EP_SF_ROW_MAJOR 0
-#define EP_SF_COL_MAJOR 1
-#define EP_SF_COL_MAJOR_COUNTED 2
-
 // One receive-stream row per wave: copy (or quantise) it into every expanded slot it owns.
 struct EpScatterArgs {
     const void* x;                // [T, hidden] rows: BF16, or FP8 bytes when prequantised
@@ -103,9 +96,26 @@ struct EpScatterArgs {
     int with_metadata;            // packed rows carry topk_idx and the source token (non-cached)
     int idx_off, w_off, src_off;  // byte offsets of the packed metadata inside a row
     int num_out_rows;             // rows of recv_x: slots outside are ignored
-    int sf_col_major;             // EP_SF_* layout of recv_sf
-    int sf_elem_bytes;            // element size of recv_sf: 2 (packs) or 4 (fp32 scales)
     int pad0;
+};
+
+// recv_sf layouts: rows of scales, or columns of scales whose stride is the row count of recv_sf
+// (EP_SF_COL_MAJOR) or the expanded row count the layout pass produced (EP_SF_COL_MAJOR_COUNTED:
+// the host does not know it yet when the kernel is enqueued).
+#define EP_SF_ROW_MAJOR 0
+#define EP_SF_COL_MAJOR 1
+#define EP_SF_COL_MAJOR_COUNTED 2
+#define EP_SF_TILE 64
+
+// Row-major scale rows -> column-major, 64 x 64 tiles through LDS.
+struct EpSfTransposeArgs {
+    const void* src;              // [num_rows, num_cols] row-major
+    void* dst;                    // column c starts at element c * (row count)
+    const int* psum_expert;       // [El]: the expanded row count is its last entry, aligned (counted layout)
+    int num_rows, num_cols;
+    int elem_bytes;               // 2 or 4
+    int counted;                  // row count and column stride come from psum_expert
+    int num_local_experts, expert_alignment;
 };
 
 // Fused single-partition combine: one receive-stream row per wave.

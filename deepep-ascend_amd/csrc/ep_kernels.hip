@@ -431,25 +431,6 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
     return true;
 }
 
-// Byte strides of recv_sf: per output row and per element column.  Column-major scales are what
-// the reference makes with a second transposing pass (csrc/buffers/ep.hpp:379-381).
-struct SfOut {
-    int64_t row, col;
-};
-__device__ __forceinline__ SfOut sf_out_strides(const EpScatterArgs& a) {
-    if (a.sf_col_major == EP_SF_ROW_MAJOR) return {a.out_sf_row_bytes, (int64_t)a.sf_elem_bytes};
-    int n = a.num_out_rows;
-    if (a.sf_col_major == EP_SF_COL_MAJOR_COUNTED)
-        n = min(n, align_up(a.psum_expert[a.num_local_experts - 1], a.expert_alignment));
-    return {(int64_t)a.sf_elem_bytes, (int64_t)n * a.sf_elem_bytes};
-}
-// Address of 2-byte pack p of row s.
-__device__ __forceinline__ unsigned short* sf_pack_ptr(const EpScatterArgs& a, const SfOut& o, int64_t s, int p) {
-    const int per_elem = a.sf_elem_bytes >> 1;
-    const int elem = per_elem == 2 ? p >> 1 : p, sub = per_elem == 2 ? p & 1 : 0;
-    return (unsigned short*)((char*)a.recv_sf + s * o.row + elem * o.col) + sub;
-}
-
 __device__ __forceinline__ void zero_padding_rows(const EpScatterArgs& a) {
     const int lane = lane_id(), w = wave_id();
     const int pb = blockIdx.x - a.num_row_blocks;
@@ -459,13 +440,13 @@ __device__ __forceinline__ void zero_padding_rows(const EpScatterArgs& a) {
     const int aend = align_up(end, a.expert_alignment);
     const int nvec = (int)(a.out_row_bytes >> 4);
     const u32x4 z = {0u, 0u, 0u, 0u};
-    SfOut so{};
-    if (a.recv_sf != nullptr) so = sf_out_strides(a);
     for (int r = end + part * EP_ROWS_PER_BLOCK + w; r < aend; r += EP_PAD_BLOCKS_PER_EXPERT * EP_ROWS_PER_BLOCK) {
         u32x4* d = (u32x4*)((char*)a.recv_x + (int64_t)r * a.out_row_bytes);
         for (int v = lane; v < nvec; v += WAVE) __builtin_nontemporal_store(z, d + v);
-        if (a.recv_sf != nullptr)
-            for (int p = lane; p < (int)(a.out_sf_row_bytes >> 1); p += WAVE) *sf_pack_ptr(a, so, r, p) = 0;
+        if (a.recv_sf != nullptr) {
+            unsigned short* s = (unsigned short*)((char*)a.recv_sf + (int64_t)r * a.out_sf_row_bytes);
+            for (int p = lane; p < (int)(a.out_sf_row_bytes >> 1); p += WAVE) s[p] = 0;
+        }
         if (a.recv_topk_weights != nullptr && lane == 0) a.recv_topk_weights[r] = 0.0f;
     }
 }
@@ -499,13 +480,12 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
     if (part == 0 && a.recv_sf != nullptr) {
         const int P = a.num_sf_packs;
         const char* sfrow = (const char*)a.sf + c.src_row * a.sf_token_stride_bytes;
-        const SfOut so = sf_out_strides(a);
         for (int p = lane; p < P; p += WAVE) {
             const unsigned short val = *(const unsigned short*)(sfrow + (int64_t)p * a.sf_pack_stride_bytes);
             for (int j = 0; j < K; ++j) {
                 const int s = readlane(c.myslot, j);
                 if (s < 0) continue;
-                *sf_pack_ptr(a, so, s, p) = val;
+                ((unsigned short*)((char*)a.recv_sf + (int64_t)s * a.out_sf_row_bytes))[p] = val;
             }
         }
     }
@@ -545,13 +525,11 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     const u32x2 q8 = quant8<HW>(f, inv);
     if (!live) return;
     const bool writes_scale = (lane & 15) == 0;
-    const SfOut so = sf_out_strides(a);
-    char* const my_scale = (char*)a.recv_sf + (int64_t)(v >> 4) * so.col;
     for (int j = 0; j < K; ++j) {
         const int s = readlane(c.myslot, j);
         if (s < 0) continue;
         __builtin_nontemporal_store(q8, (u32x2*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes) + v);
-        if (writes_scale) *(float*)(my_scale + (int64_t)s * so.row) = scale;
+        if (writes_scale) ((float*)((char*)a.recv_sf + (int64_t)s * a.out_sf_row_bytes))[v >> 4] = scale;
     }
 }
 
@@ -560,6 +538,38 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant(Ep
 }
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_sw(EpScatterArgs a) {
     scatter_quant_body<false>(a);
+}
+
+// Column-major scales (use_tma_aligned_col_major_sf): the copy kernels write scale rows, this
+// kernel turns them into columns.  The reference does the same with a generic transposing copy
+// (csrc/buffers/ep.hpp:379-381); writing columns straight from the copy kernel was measured and is
+// slower, since every 4-byte scale then lands in a cache line of its own.
+template <typename E>
+__device__ __forceinline__ void sf_transpose_body(const EpSfTransposeArgs& a, unsigned (*tile)[EP_SF_TILE + 1]) {
+    int n = a.num_rows;
+    if (a.counted) n = min(n, align_up(a.psum_expert[a.num_local_experts - 1], a.expert_alignment));
+    const int r0 = blockIdx.x * EP_SF_TILE;
+    if (r0 >= n) return;
+    const int tx = threadIdx.x % EP_SF_TILE, ty = threadIdx.x / EP_SF_TILE;
+    constexpr int STEP = EP_LAYOUT_THREADS / EP_SF_TILE;
+    const E* src = (const E*)a.src;
+    E* dst = (E*)a.dst;
+    for (int c0 = 0; c0 < a.num_cols; c0 += EP_SF_TILE) {
+        for (int rr = ty; rr < EP_SF_TILE; rr += STEP)
+            if (r0 + rr < n && c0 + tx < a.num_cols) tile[rr][tx] = src[(int64_t)(r0 + rr) * a.num_cols + c0 + tx];
+        __syncthreads();
+        for (int cc = ty; cc < EP_SF_TILE; cc += STEP)
+            if (c0 + cc < a.num_cols && r0 + tx < n) dst[(int64_t)(c0 + cc) * n + r0 + tx] = (E)tile[tx][cc];
+        __syncthreads();
+    }
+}
+
+extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_sf_transpose(EpSfTransposeArgs a) {
+    __shared__ unsigned tile[EP_SF_TILE][EP_SF_TILE + 1];
+    if (a.elem_bytes == 4)
+        sf_transpose_body<unsigned>(a, tile);
+    else
+        sf_transpose_body<unsigned short>(a, tile);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -109,7 +109,7 @@ int64_t combine_buffer_size(int ranks, int max_tokens, int hidden, int topk) {
 struct Kernels {
     hipModule_t module = nullptr;
     hipFunction_t layout_count, layout_scan, layout_assign;
-    hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw;
+    hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw, sf_transpose;
     hipFunction_t combine[3][5];     // [mode][generic, k2, k4, k6, k8]
     hipFunction_t fp8_selftest;
     int device = -1;
@@ -147,6 +147,7 @@ void load_kernels(const char* dir) {
     get(g_k.scatter_copy, "ep_scatter_copy");
     get(g_k.scatter_quant, "ep_scatter_quant");
     get(g_k.scatter_quant_sw, "ep_scatter_quant_sw");
+    get(g_k.sf_transpose, "ep_sf_transpose");
     const char* modes[3] = {"", "_partial", "_final"};
     const char* ks[5] = {"_generic", "_k2", "_k4", "_k6", "_k8"};
     for (int mode = 0; mode < 3; ++mode)
@@ -474,8 +475,6 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             sa.copy_bytes = sa.x_row_bytes;
             sa.out_row_bytes = pk.bytes;
             sa.out_sf_row_bytes = pk.bytes;
-            sa.sf_col_major = EP_SF_ROW_MAJOR;
-            sa.sf_elem_bytes = a.fused_fp8_quant ? 4 : 2;
             if (present(a.sf)) {
                 sa.sf_token_stride_bytes = a.sf.stride[0] * 2;
                 sa.sf_pack_stride_bytes = a.sf.stride[1] * 2;
@@ -640,10 +639,16 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
             // row-major scale rows (csrc/kernels/ep/dispatch.hpp:112-113), or the column-major result of
             // the reference's transposing pass (csrc/buffers/ep.hpp:379-381) written in place
             EP_HOST_ASSERT(a.recv_sf_layout >= EP_SF_ROW_MAJOR and a.recv_sf_layout <= EP_SF_COL_MAJOR_COUNTED);
-            if (a.recv_sf_layout == EP_SF_ROW_MAJOR)
+            if (a.recv_sf_layout == EP_SF_ROW_MAJOR) {
                 EP_HOST_ASSERT(a.recv_sf.stride[1] == 1 and a.recv_sf.stride[0] == a.recv_sf.size[1]);
-            else
+            } else {
                 EP_HOST_ASSERT(a.recv_sf.stride[0] == 1 and a.recv_sf.stride[1] == a.recv_sf.size[0]);
+                // the copy kernel writes scale rows into the staging tensor, a second kernel turns them
+                const ep_tensor_t& st = a.recv_sf_staging;
+                EP_HOST_ASSERT(present(st) and st.ndim == 2 and st.dtype == a.recv_sf.dtype);
+                EP_HOST_ASSERT(st.size[0] == a.recv_sf.size[0] and st.size[1] == a.recv_sf.size[1]);
+                EP_HOST_ASSERT(st.stride[1] == 1 and st.stride[0] == st.size[1] and st.data != a.recv_sf.data);
+            }
         }
         if (present(a.topk_weights)) {
             EP_HOST_ASSERT(present(a.recv_topk_weights) and a.recv_topk_weights.ndim == 1);
@@ -668,13 +673,12 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.num_recv_ptr = (const int*)a.psum_num_recv_tokens_per_rank.data + (R - 1);
         sa.recv_src_metadata = (int*)a.recv_src_metadata.data;
         sa.recv_x = a.recv_x.data;
-        sa.recv_sf = has_sf ? a.recv_sf.data : nullptr;
+        const bool sf_columns = has_sf and a.recv_sf_layout != EP_SF_ROW_MAJOR;
+        sa.recv_sf = has_sf ? (sf_columns ? a.recv_sf_staging.data : a.recv_sf.data) : nullptr;
         sa.recv_topk_weights = present(a.topk_weights) ? (float*)a.recv_topk_weights.data : nullptr;
         sa.psum_expert = (const int*)a.psum_num_recv_tokens_per_expert.data;
         sa.out_row_bytes = (int64_t)hidden * elem_size(a.recv_x.dtype);
         sa.out_sf_row_bytes = has_sf ? a.recv_sf.size[1] * elem_size(a.recv_sf.dtype) : 0;
-        sa.sf_elem_bytes = has_sf ? elem_size(a.recv_sf.dtype) : 2;
-        sa.sf_col_major = has_sf ? a.recv_sf_layout : EP_SF_ROW_MAJOR;
         sa.hidden = hidden;
         sa.num_topk = K;
         // never walk past the rows the metadata tensor holds
@@ -724,9 +728,23 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0);
         const unsigned pad_blocks = a.do_zero_padding ? (unsigned)El * EP_PAD_BLOCKS_PER_EXPERT : 0u;
         const unsigned grid = (unsigned)sa.num_row_blocks + pad_blocks;
-        if (grid == 0) return;
-        hipFunction_t fn = quantise_here ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
-        launch(fn, grid, EP_ROW_THREADS, 0, a.stream, sa);
+        if (grid > 0) {
+            hipFunction_t fn = quantise_here ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
+            launch(fn, grid, EP_ROW_THREADS, 0, a.stream, sa);
+        }
+        if (sf_columns and num_expanded > 0) {
+            EpSfTransposeArgs ta{};
+            ta.src = a.recv_sf_staging.data;
+            ta.dst = a.recv_sf.data;
+            ta.psum_expert = sa.psum_expert;
+            ta.num_rows = sa.num_out_rows;
+            ta.num_cols = (int)a.recv_sf.size[1];
+            ta.elem_bytes = elem_size(a.recv_sf.dtype);
+            ta.counted = a.recv_sf_layout == EP_SF_COL_MAJOR_COUNTED ? 1 : 0;
+            ta.num_local_experts = El;
+            ta.expert_alignment = a.expert_alignment;
+            launch(g_k.sf_transpose, (unsigned)ceil_div(ta.num_rows, EP_SF_TILE), EP_LAYOUT_THREADS, 0, a.stream, ta);
+        }
     });
 }
 

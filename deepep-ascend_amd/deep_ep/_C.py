@@ -43,7 +43,7 @@ class _DispatchArgs(ctypes.Structure):
 class _DispatchEpilogueArgs(ctypes.Structure):
     _fields_ = [(n, _Tensor) for n in (
         'x', 'sf', 'topk_weights', 'psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
-        'recv_x', 'recv_sf', 'recv_topk_weights', 'recv_src_metadata')] + [
+        'recv_x', 'recv_sf', 'recv_sf_staging', 'recv_topk_weights', 'recv_src_metadata')] + [
         ('num_topk', ctypes.c_int32), ('num_max_tokens_per_rank', ctypes.c_int32), ('num_experts', ctypes.c_int32),
         ('expert_alignment', ctypes.c_int32), ('cached_mode', ctypes.c_int32), ('do_zero_padding', ctypes.c_int32),
         ('fused_fp8_quant', ctypes.c_int32), ('recv_sf_layout', ctypes.c_int32), ('stream', ctypes.c_void_p)]
@@ -415,8 +415,10 @@ class EPBuffer(BufferBase):
             if fused_fp8_quant or sf is not None:
                 sf_cols = (hidden + 127) // 128 if fused_fp8_quant else sf.size(1)
                 sf_dtype = torch.float32 if fused_fp8_quant else sf.dtype
+                sf_staging = None
                 if use_col_major_sf:
-                    # the copy kernel writes the scales column by column: no transposing pass afterwards
+                    # scale rows go to a staging tensor, a tiled kernel of the library turns them into columns
+                    sf_staging = torch.empty((alloc_expanded, sf_cols), dtype=sf_dtype, device=dev)
                     sf_storage = torch.empty((sf_cols * alloc_expanded,), dtype=sf_dtype, device=dev)
                     recv_sf = sf_storage.as_strided((alloc_expanded, sf_cols), (1, alloc_expanded))
                 else:
@@ -436,6 +438,8 @@ class EPBuffer(BufferBase):
             e.psum_num_recv_tokens_per_rank = a.psum_num_recv_tokens_per_rank
             e.psum_num_recv_tokens_per_expert = a.psum_num_recv_tokens_per_expert
             e.recv_x, e.recv_sf = _desc(recv_x), _desc(recv_sf, two_byte_packs=not fused_fp8_quant)
+            if recv_sf is not None:
+                e.recv_sf_staging = _desc(sf_staging, two_byte_packs=not fused_fp8_quant)
             e.recv_topk_weights, e.recv_src_metadata = _desc(recv_topk_weights), _desc(recv_src_metadata)
             e.num_topk, e.num_max_tokens_per_rank = num_topk, num_max_tokens_per_rank
             e.num_experts, e.expert_alignment = num_experts, expert_alignment

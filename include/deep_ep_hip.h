@@ -126,15 +126,17 @@ typedef struct ep_dispatch_epilogue_args {
     ep_tensor_t psum_num_recv_tokens_per_rank, psum_num_recv_tokens_per_expert;
     ep_tensor_t recv_x;                                 /* [N_exp,H] out, dtype of x (FP8 if fused) */
     ep_tensor_t recv_sf;                                /* [N_exp,P] out, laid out as recv_sf_layout says */
+    ep_tensor_t recv_sf_staging;                        /* [N_exp,P] row-major scratch; layouts 1 and 2 only */
     ep_tensor_t recv_topk_weights;                      /* [N_exp] fp32 out (optional) */
     ep_tensor_t recv_src_metadata;                      /* [N_recv,K+2] int32: out, or in when cached */
     int32_t num_topk, num_max_tokens_per_rank, num_experts, expert_alignment;
     int32_t cached_mode, do_zero_padding, fused_fp8_quant;
     /* 0: rows of scales, strides (P,1) (ep.hpp:328-336).  1: columns of scales, strides (1,N_exp): the
-     * layout the reference reaches with a second transposing pass (ep.hpp:379-381), written here by
-     * the copy kernel itself.  2: as 1, but recv_sf describes storage for an upper bound of rows and
-     * the column stride is the expanded row count of this dispatch, read on the device: the result
-     * is the tensor of shape (N_exp,P), strides (1,N_exp) at the start of that storage. */
+     * layout the reference reaches with a transposing copy after its epilogue (ep.hpp:379-381); here
+     * the copy kernel writes scale rows into recv_sf_staging and a tiled kernel turns them into
+     * recv_sf.  2: as 1, but recv_sf describes storage for an upper bound of rows and the column
+     * stride is the expanded row count of this dispatch, read on the device: the result is the
+     * tensor of shape (N_exp,P), strides (1,N_exp) at the start of that storage. */
     int32_t recv_sf_layout;
     void* stream;
 } ep_dispatch_epilogue_args_t;

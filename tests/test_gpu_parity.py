@@ -167,7 +167,7 @@ def test_fp8_dispatch_fused_and_prequantised(T, H, E, K, A, masked, zipf):
 
 @pytest.mark.parametrize('R,rank', [(1, 0), (4, 2)])
 @pytest.mark.parametrize('do_cpu_sync', [True, False])
-def test_column_major_scales_are_written_in_place(R, rank, do_cpu_sync):
+def test_column_major_scales(R, rank, do_cpu_sync):
     """use_tma_aligned_col_major_sf: strides (1, N) exactly as the reference's transposing pass leaves
     them (tests/ep/test_ep.py:141-145), for fused and pre-quantised input, with and without the host
     sync, for a cached replay, and at R > 1 where fp32 scales travel as two 2-byte packs."""
