@@ -178,9 +178,15 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--cpu-sample-tokens', type=int, default=16384)
     ap.add_argument('--no-cpu-sync', action='store_true', help='dispatch without the host count wait')
+    ap.add_argument('--graph', action='store_true',
+                    help='record the step (dispatch without host sync + combine) into a HIP graph and replay it')
+    ap.add_argument('--no-flush', action='store_true',
+                    help='per-kernel samples back to back, without rewriting a 1 GiB scratch buffer between them')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run a plain 1 GiB device copy (known traffic) to scale rocprof byte counters')
     args = ap.parse_args()
+    if args.graph:
+        args.no_cpu_sync = True     # a graph cannot hold the host's wait for the counts
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py measures one GPU\'s share of the EP path; run it with --gpus 1 (no collectives exist here)',
               file=sys.stderr)
@@ -228,20 +234,36 @@ def main():
         r, _, rw, h, _ = dispatch()
         buf.combine(y, h, topk_weights=rw)
 
+    run_step = step
+    if args.graph:
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        run_step = graph.replay
     for _ in range(args.warmup):
-        step()
+        run_step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run_step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # per-kernel durations with events on the launch stream (the current stream): the copy kernel alone
     # is what a cached dispatch enqueues, the combine is a single kernel, the layout is the remainder
+    # Between samples a 1 GiB scratch buffer is rewritten, so no sample finds its inputs in the L2 or
+    # the memory-side cache (the reference's benchmark does the same: tests/ep/test_ep.py:79-80,415-421).
+    scratch = None if args.no_flush else torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+
     def timed(fn, n):
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
         for a, b in evs:
+            if scratch is not None:
+                scratch.zero_()
             a.record()
             fn()
             b.record()
@@ -253,16 +275,19 @@ def main():
     t_combine = timed(lambda: buf.combine(y, handle, topk_weights=recv_w), n_k)
     t_dispatch_full = timed(lambda: dispatch(), n_k)
     avg = lambda v: sum(v) / len(v)  # noqa: E731
+    med = lambda v: v[len(v) // 2]  # noqa: E731
     us_scatter, us_combine, us_dispatch = avg(t_scatter), avg(t_combine), avg(t_dispatch_full)
 
-    def roof(name, nbytes, us):
+    def roof(name, nbytes, samples):
+        us = avg(samples)
         gbs = nbytes / us / 1e3
         traffic = MEASURED_TRAFFIC.get((args.workload, name)) if not args.no_cpu_sync else None
         return {'kernel': name, 'bound': 'hbm', 'achieved': round(gbs, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': round(gbs / HBM_PEAK_GBS, 4), 'traffic': traffic, 'us': round(us, 2), 'bytes': nbytes}
+                'frac': round(gbs / HBM_PEAK_GBS, 4), 'traffic': traffic, 'us': round(us, 2),
+                'us_median': round(med(samples), 2), 'bytes': nbytes}
 
     scatter_name = 'ep_scatter_quant' if fp8 else 'ep_scatter_copy'
-    kernels = [roof(scatter_name, b_d, us_scatter), roof(f'ep_combine_k{K}', b_c, us_combine)]
+    kernels = [roof(scatter_name, b_d, t_scatter), roof(f'ep_combine_k{K}', b_c, t_combine)]
     dominant = max(kernels, key=lambda k: k['us'])
     out = {
         'metric': 'dispatch & combine GB/s + % of HBM peak, 16384 tok x7168, top-6/256, FP8/BF16',
@@ -274,7 +299,8 @@ def main():
         'config': {'workload': args.workload, 'tokens': T, 'hidden': H, 'experts': E, 'topk': K,
                    'expert_alignment': A, 'partitions': 1, 'dispatch': 'fused bf16->fp8 e4m3 + per-128 fp32 scales'
                    if fp8 else 'bf16', 'combine': 'bf16, fp32 accumulate, weights carried back, no bias',
-                   'do_zero_padding': True, 'do_cpu_sync': not args.no_cpu_sync,
+                   'do_zero_padding': True, 'do_cpu_sync': not args.no_cpu_sync, 'hip_graph': bool(args.graph),
+                   'cache_flush_between_kernel_samples': not args.no_flush,
                    'num_valid_rows': n_valid, 'num_expanded_rows': n_exp_exact},
         'roofline': {k: dominant[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'traffic')} |
                     {'kernel': dominant['kernel']},

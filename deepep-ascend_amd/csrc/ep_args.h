@@ -12,7 +12,7 @@
 #define EP_SCAN_THREADS 1024
 #define EP_ROW_THREADS 256        // 4 waves, one row per wave
 #define EP_ROWS_PER_BLOCK 4
-#define EP_PAD_BLOCKS_PER_EXPERT 4
+#define EP_MAX_PAD_BLOCKS_PER_EXPERT 16
 
 #define EP_LAYOUT_SCANNED 0
 #define EP_LAYOUT_SINGLE 2
@@ -96,7 +96,7 @@ struct EpScatterArgs {
     int with_metadata;            // packed rows carry topk_idx and the source token (non-cached)
     int idx_off, w_off, src_off;  // byte offsets of the packed metadata inside a row
     int num_out_rows;             // rows of recv_x: slots outside are ignored
-    int pad0;
+    int pad_blocks_per_expert;    // workgroups that share the zeroing of one expert's padding rows
 };
 
 // recv_sf layouts: rows of scales, or columns of scales whose stride is the row count of recv_sf

@@ -431,24 +431,34 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
     return true;
 }
 
+// The padding rows of an expert, [psum[e], align(psum[e], A)), are one contiguous span of each output:
+// the workgroups that share it walk the span 4 KiB at a time, 16 bytes per lane
+// (dispatch_copy_epilogue.hpp:547-620).
+__device__ __forceinline__ void zero_span(char* base, int64_t nbytes, int part, int nparts) {
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    const int64_t tid = (int64_t)part * EP_ROW_THREADS + threadIdx.x;     // among the threads sharing the span
+    const int64_t nthreads = (int64_t)nparts * EP_ROW_THREADS;
+    // 16-byte stores over the aligned body; the ends in 2-byte units (every element here is 2 or 4 bytes wide)
+    const int64_t head = min((int64_t)((16 - ((uintptr_t)base & 15)) & 15), nbytes);
+    const int64_t body = (nbytes - head) & ~(int64_t)15;
+    for (int64_t o = tid * 16; o < body; o += nthreads * 16) __builtin_nontemporal_store(z, (u32x4*)(base + head + o));
+    for (int64_t o = tid * 2; o < head; o += nthreads * 2) *(unsigned short*)(base + o) = 0;
+    for (int64_t o = head + body + tid * 2; o < nbytes; o += nthreads * 2) *(unsigned short*)(base + o) = 0;
+}
+
 __device__ __forceinline__ void zero_padding_rows(const EpScatterArgs& a) {
-    const int lane = lane_id(), w = wave_id();
     const int pb = blockIdx.x - a.num_row_blocks;
-    const int e = pb / EP_PAD_BLOCKS_PER_EXPERT, part = pb % EP_PAD_BLOCKS_PER_EXPERT;
+    const int e = pb / a.pad_blocks_per_expert, part = pb % a.pad_blocks_per_expert;
     if (e >= a.num_local_experts) return;
     const int end = a.psum_expert[e];
-    const int aend = align_up(end, a.expert_alignment);
-    const int nvec = (int)(a.out_row_bytes >> 4);
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    for (int r = end + part * EP_ROWS_PER_BLOCK + w; r < aend; r += EP_PAD_BLOCKS_PER_EXPERT * EP_ROWS_PER_BLOCK) {
-        u32x4* d = (u32x4*)((char*)a.recv_x + (int64_t)r * a.out_row_bytes);
-        for (int v = lane; v < nvec; v += WAVE) __builtin_nontemporal_store(z, d + v);
-        if (a.recv_sf != nullptr) {
-            unsigned short* s = (unsigned short*)((char*)a.recv_sf + (int64_t)r * a.out_sf_row_bytes);
-            for (int p = lane; p < (int)(a.out_sf_row_bytes >> 1); p += WAVE) s[p] = 0;
-        }
-        if (a.recv_topk_weights != nullptr && lane == 0) a.recv_topk_weights[r] = 0.0f;
-    }
+    const int rows = align_up(end, a.expert_alignment) - end;
+    if (rows <= 0) return;
+    zero_span((char*)a.recv_x + (int64_t)end * a.out_row_bytes, (int64_t)rows * a.out_row_bytes, part,
+              a.pad_blocks_per_expert);
+    if (a.recv_sf != nullptr && part == 0)
+        zero_span((char*)a.recv_sf + (int64_t)end * a.out_sf_row_bytes, (int64_t)rows * a.out_sf_row_bytes, 0, 1);
+    if (a.recv_topk_weights != nullptr && part == a.pad_blocks_per_expert - 1)
+        zero_span((char*)(a.recv_topk_weights + end), (int64_t)rows * 4, 0, 1);
 }
 
 // Verbatim rows: BF16 payload, or FP8 payload with its 2-byte scale packs.  A task moves 1 KiB of

@@ -726,7 +726,9 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.num_parts = (int)std::max<int64_t>(1, quantise_here ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024));
         sa.num_row_blocks = (int)ceil_div((int64_t)sa.num_rows_bound * sa.num_parts, EP_ROWS_PER_BLOCK);
         EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0);
-        const unsigned pad_blocks = a.do_zero_padding ? (unsigned)El * EP_PAD_BLOCKS_PER_EXPERT : 0u;
+        // an expert has at most alignment - 1 padding rows: about one workgroup per 8 of them
+        sa.pad_blocks_per_expert = std::max(1, std::min(EP_MAX_PAD_BLOCKS_PER_EXPERT, a.expert_alignment / 8));
+        const unsigned pad_blocks = a.do_zero_padding ? (unsigned)(El * sa.pad_blocks_per_expert) : 0u;
         const unsigned grid = (unsigned)sa.num_row_blocks + pad_blocks;
         if (grid > 0) {
             hipFunction_t fn = quantise_here ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
