@@ -30,6 +30,13 @@
 //   [1] number of received tokens   [2] number of expanded tokens (aligned)
 //   [16 .. 16+R)                 received tokens per source rank
 //   [16+EP_MAX_RANKS .. +El)     aligned received tokens per local expert
+// Fixed header of every arena's workspace; the layout scratch is carved behind it.
+//   [0, 4*EP_MAX_RANKS)                    inbox: rows each source partition put into this partition's regions
+//   [EP_WS_PEERS_OFF, +8*EP_MAX_RANKS)     arena base of every partition of the node (own arena when not connected)
+#define EP_WS_INBOX_OFF 0
+#define EP_WS_PEERS_OFF 1024
+#define EP_WS_HEADER_BYTES 4096
+
 #define EP_HOST_RANK_OFF 16
 #define EP_HOST_EXPERT_OFF (16 + EP_MAX_RANKS)
 #define EP_HOST_PAGE_INTS (16 + EP_MAX_RANKS + EP_MAX_EXPERTS)
@@ -57,6 +64,17 @@ struct EpLayoutArgs {
     int* unaligned_expert;        // [El]
     int* cumulative_stats;        // [El] or null
     int* host_page;               // device view of the mapped host page
+    // partitioned path (more than one partition)
+    int send_only;                // send side: only dst_buffer_slot_idx / dst_gsge_idx and the peers' inboxes are written
+    int recv_mode;                // receive side: the entries are the rows that arrived in this partition's regions
+    char* const* peer_arenas;     // [R] arena bases (send side: whose inbox gets this partition's row counts)
+    const int* inbox;             // [R] rows per source (receive side)
+    const char* packed_base;      // this partition's regions of packed rows (receive side)
+    int64_t packed_row_bytes;
+    int idx_off, src_off;         // byte offsets of topk_idx and of the source token inside a packed row
+    int* recv_src_metadata;       // [rows_cap, K+2]  (receive side: written here, there is no slot_map)
+    int rows_cap;                 // rows the metadata tensor holds
+    int connected;                // the peers are arenas of their own (a node), not this arena again
 };
 
 // One receive-stream row per wave: copy (or quantise) it into every expanded slot it owns.
@@ -91,12 +109,20 @@ struct EpScatterArgs {
     const int64_t* topk_idx;      // [T, K]            (pack)
     const int* dst_slot_idx;      // [T, K]            (pack)
     int64_t copy_bytes;           // payload bytes moved per row (verbatim kernel)
-    int64_t src_base_row;         // first packed row of this partition's own region (region mode)
     int num_experts, experts_per_rank;
     int with_metadata;            // packed rows carry topk_idx and the source token (non-cached)
     int idx_off, w_off, src_off;  // byte offsets of the packed metadata inside a row
     int num_out_rows;             // rows of recv_x: slots outside are ignored
     int pad_blocks_per_expert;    // workgroups that share the zeroing of one expert's padding rows
+    // where packed rows go (pack) and come from (region): partition p's regions start at
+    // peer_arenas[p] + buffer_off; a row for partition r lands in region `region_by_source ? rank_idx : r`
+    char* const* peer_arenas;
+    const int* psum_rank;         // [R] inclusive row counts per source (region mode: stream row -> region, slot)
+    int64_t buffer_off;
+    int region_by_source;
+    int num_ranks;
+    int pack_sf_off;              // byte offset of the scales inside a packed row (pack mode)
+    int pad2;
 };
 
 // recv_sf layouts: rows of scales, or columns of scales whose stride is the row count of recv_sf
@@ -140,6 +166,9 @@ struct EpCombineArgs {
     int num_ranks, experts_per_rank;
     int num_in_rows;              // rows of y: slots outside are ignored
     int num_groups;               // partial groups of the combine buffer: min(K, R)
+    // owner-side reduce: the partial of a row goes to the combine buffer of the partition its token came from
+    char* const* peer_arenas;
+    int64_t buffer_off;
 };
 
 // Hardware vs integer e4m3fn conversion over fp32 bit patterns [first, first+count).

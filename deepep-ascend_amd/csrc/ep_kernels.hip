@@ -49,9 +49,57 @@ __device__ __forceinline__ int wave_inclusive_sum(int v) {
 // Layout pass A: per-block histograms of expert ids and of destination-partition masters.
 // Reference semantics: impls/ep/dispatch.hpp:166-194 (expert histogram, dedup by partition).
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s_key, short* s_rk) {
+// Receive side: inclusive row counts per source partition from the inbox, in LDS.  Every thread of
+// the workgroup calls it (blockDim >= R); returns the length of the receive stream.  s_psum holds
+// R + blockDim/64 ints.
+__device__ __forceinline__ int recv_scan_sources(const EpLayoutArgs& a, int* s_psum) {
+    const int R = a.num_ranks, tid = threadIdx.x, lane = lane_id(), w = wave_id();
+    int* s_w = s_psum + R;
+    int v = 0;
+    if (tid < R) v = max(0, min(a.inbox[tid], a.max_tokens));
+    const int incl = wave_inclusive_sum(v);
+    if (lane == WAVE - 1) s_w[w] = incl;
+    __syncthreads();
+    int off = 0;
+    for (int i = 0; i < w; ++i) off += s_w[i];
+    if (tid < R) s_psum[tid] = off + incl;
+    __syncthreads();
+    return s_psum[R - 1];
+}
+
+// Row g of the receive stream (the regions of the source partitions one after the other, each up to
+// its row count: the PSumIterator of dispatch_copy_epilogue.hpp:130-174) -> packed row index.
+__device__ __forceinline__ int64_t recv_packed_row(const int* psum, int R, int max_tokens, int g) {
+    int lo = 0, hi = R - 1;                       // first source whose inclusive count exceeds g
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (psum[mid] > g) hi = mid; else lo = mid + 1;
+    }
+    return (int64_t)lo * max_tokens + (g - (lo ? psum[lo - 1] : 0));
+}
+
+// Stages the expert ids of this workgroup's entries.  Send side: entry (t, j) of topk_idx.  Receive
+// side: entry (row, j) of the receive stream, read from the packed row; partitions play no role there.
+// Returns the number of rows (tokens) the entries range over.
+__device__ __forceinline__ int layout_load_keys(const EpLayoutArgs& a, short* s_key, short* s_rk, int* s_psum) {
     const int K = a.num_topk;
     const int n = EP_TOKENS_PER_BLOCK * K;
+    if (a.recv_mode) {
+        const int N = recv_scan_sources(a, s_psum);
+        for (int i = threadIdx.x; i < n; i += blockDim.x) {
+            const int row = i / K, j = i - row * K;
+            const int g = blockIdx.x * EP_TOKENS_PER_BLOCK + row;
+            int e = -1;
+            if (g < N) {
+                const int64_t pr = recv_packed_row(s_psum, a.num_ranks, a.max_tokens, g);
+                const int64_t v = ((const int64_t*)(a.packed_base + pr * a.packed_row_bytes + a.idx_off))[j];
+                e = (v >= 0 && v < a.num_experts) ? (int)v : -1;
+            }
+            s_key[i] = (short)e;
+            s_rk[i] = -1;
+        }
+        return N;
+    }
     const int64_t base = (int64_t)blockIdx.x * n;
     const int64_t total = (int64_t)a.num_tokens * K;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -63,6 +111,7 @@ __device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s
         s_key[i] = (short)e;
         s_rk[i] = (short)(e < 0 ? -1 : e / a.experts_per_rank);
     }
+    return a.num_tokens;
 }
 
 // Destination partition of entry idx if it is the last slot of its token going there, else -1
@@ -83,8 +132,9 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(
     int* s_rcnt = s_ecnt + E;           // [R]
     short* s_key = (short*)(s_rcnt + R);
     short* s_rk = s_key + EP_TOKENS_PER_BLOCK * K;
+    int* s_psum = (int*)(s_rk + EP_TOKENS_PER_BLOCK * K);      // [R + waves]  (receive side)
     for (int i = threadIdx.x; i < E + R; i += blockDim.x) smem[i] = 0;
-    layout_load_keys(a, s_key, s_rk);
+    layout_load_keys(a, s_key, s_rk, s_psum);
     __syncthreads();
     const int n = EP_TOKENS_PER_BLOCK * K;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -170,13 +220,14 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     int* s_tmp = s_wr + NW * R;            // [NW + 1]
     short* s_key = (short*)(s_tmp + NW + 1);
     short* s_rk = s_key + EP_TOKENS_PER_BLOCK * K;
+    int* s_psum = (int*)(s_rk + EP_TOKENS_PER_BLOCK * K);      // [R + NW]  (receive side)
     const int tid = threadIdx.x, lane = lane_id(), w = wave_id();
     const int lo = a.rank_idx * El;
     const int ncols = El + R;              // column c < El: local expert lo + c; else partition c - El
 
     // ---- A: stage this block's keys, clear the per-wave counters ----
     for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
-    layout_load_keys(a, s_key, s_rk);
+    const int num_rows = layout_load_keys(a, s_key, s_rk, s_psum);
     __syncthreads();
 
     // ---- B: per-wave counts: wave w owns entries [w*epw, (w+1)*epw) of this block's chunk ----
@@ -235,7 +286,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
         int run = wave_off + incl - mine;
         for (int e = e0; e < e1; ++e) {
             const int c = s_tot[e];
-            if (b == 0) {
+            if (b == 0 && !a.send_only) {
                 a.unaligned_expert[e] = c;
                 a.psum_expert[e] = run + c;
                 if (a.cumulative_stats != nullptr) atomicAdd(&a.cumulative_stats[e], c);
@@ -245,17 +296,29 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             run += align_up(c, A);
         }
     }
-    if (b == 0) {
-        const int n_self = s_tot[El + a.rank_idx];
+    if (b == 0 && a.send_only) {
+        // rows this partition sends to every partition, left in the receivers' inboxes: the count half of
+        // the reference's cross-rank reduction (impls/ep/dispatch.hpp:469-545)
+        // (a partition that is not connected to a node only has its own inbox)
+        for (int r = tid; r < R; r += blockDim.x)
+            if (a.connected || r == a.rank_idx)
+                ((int*)(a.peer_arenas[r] + EP_WS_INBOX_OFF))[a.rank_idx] = min(s_tot[El + r], a.max_tokens);
+    }
+    if (b == 0 && !a.send_only) {
+        // one partition: the receive stream is this partition's own routed tokens; several: the rows counted
+        // in the inbox (csrc/buffers/ep.hpp:205-246 names the tensors)
+        const int n_recv = a.recv_mode ? num_rows : s_tot[El + a.rank_idx];
         for (int r = tid; r < R; r += blockDim.x) {
-            a.psum_rank[r] = r >= a.rank_idx ? n_self : 0;
-            if (a.notify_host) a.host_page[EP_HOST_RANK_OFF + r] = r == a.rank_idx ? n_self : 0;
+            const int upto = a.recv_mode ? s_psum[r] : n_recv;
+            const int from = a.recv_mode && r ? s_psum[r - 1] : 0;
+            a.psum_rank[r] = upto;
+            if (a.notify_host) a.host_page[EP_HOST_RANK_OFF + r] = upto - from;
         }
         if (a.notify_host) {
             __threadfence_system();
             __syncthreads();
             if (tid == 0) {
-                a.host_page[1] = n_self;
+                a.host_page[1] = n_recv;
                 a.host_page[2] = grand;
                 __threadfence_system();
                 __hip_atomic_store(&a.host_page[0], a.seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -285,7 +348,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     const int ebits = 32 - __builtin_clz(E);       // keys+1 in [0, E]
     const int rbits = 32 - __builtin_clz(R);
     const uint64_t lt = (1ull << lane) - 1ull;
-    const int64_t total = (int64_t)a.num_tokens * K;
+    const int64_t total = (int64_t)num_rows * K;
     for (int rd = 0; rd < rounds; ++rd) {
         const int idx = w * epw + rd * WAVE + lane;
         const bool in = idx < n;
@@ -306,14 +369,38 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
         }
         const int64_t g = (int64_t)b * n + idx;
         if (in && g < total) {
-            a.dst_buffer_slot_idx[g] = rslot;
-            a.dst_gsge_idx[g] = -1;                 // every copy is local: no transport descriptors
-            a.slot_map[g] = eslot;
-            if (mr == a.rank_idx && rslot < a.max_tokens) a.recv_tok[rslot] = b * EP_TOKENS_PER_BLOCK + idx / K;
+            if (a.recv_mode) {
+                const int64_t row = g / K;
+                if (row < a.rows_cap) a.recv_src_metadata[row * (K + 2) + (g - row * K)] = eslot;
+            } else {
+                a.dst_buffer_slot_idx[g] = rslot;
+                a.dst_gsge_idx[g] = -1;             // every copy is local: no transport descriptors
+                if (!a.send_only) {
+                    a.slot_map[g] = eslot;
+                    if (mr == a.rank_idx && rslot < a.max_tokens) a.recv_tok[rslot] = b * EP_TOKENS_PER_BLOCK + idx / K;
+                }
+            }
         }
         // the running counters of a wave are touched by that wave only and the LDS operations of a wave
         // complete in order: no block barrier (which would also wait for the stores above) is needed
         __builtin_amdgcn_wave_barrier();
+    }
+    if (a.recv_mode) {
+        // the two trailing columns of the metadata rows: source token and last local selection
+        // (dispatch_copy_epilogue.hpp:514-522)
+        for (int row = tid; row < EP_TOKENS_PER_BLOCK; row += blockDim.x) {
+            const int g = b * EP_TOKENS_PER_BLOCK + row;
+            if (g >= num_rows || g >= a.rows_cap) continue;
+            int master = -1;
+            for (int j = 0; j < K; ++j) {
+                const int le = s_key[row * K + j] - lo;
+                if (le >= 0 && le < El) master = j;
+            }
+            const int64_t pr = recv_packed_row(s_psum, R, a.max_tokens, g);
+            int* m = a.recv_src_metadata + (int64_t)g * (K + 2);
+            m[K] = *(const int*)(a.packed_base + pr * a.packed_row_bytes + a.src_off);
+            m[K + 1] = master;
+        }
     }
 }
 
@@ -355,10 +442,35 @@ __device__ __forceinline__ u32x2 quant8(const float* f, float inv) {
 }
 
 struct RowCtx {
-    int t;            // local token index of the row
+    int t;            // local token index of the row (expand and pack)
     int myslot;       // lane j < K: destination row of (row, j) or -1
+    uint64_t mybase;  // lane j < K: first byte of the regions that row belongs to (pack)
     int64_t src_row;  // row of the source matrix holding the payload
 };
+
+// Stream row i of the receive side -> packed row of this partition's regions, with the inclusive row
+// counts per source in global memory.  Every lane of the wave calls it.
+__device__ __forceinline__ int64_t region_row_of_stream(const int* psum, int R, int max_tokens, int i) {
+    const int lane = lane_id();
+    int q = 0;                                         // sources whose rows all come before row i
+    for (int r0 = 0; r0 < R; r0 += WAVE) {
+        const bool before = r0 + lane < R && psum[r0 + lane] <= i;
+        q += __popcll(__ballot(before));
+    }
+    q = min(q, R - 1);
+    return (int64_t)q * max_tokens + (i - (q ? psum[q - 1] : 0));
+}
+
+// First byte of the rows that destination j of the task writes, and of their scales.
+__device__ __forceinline__ char* out_rows_of(const EpScatterArgs& a, const RowCtx& c, int j) {
+    if (a.mode != EP_SCATTER_PACK) return (char*)a.recv_x;
+    const unsigned lo = (unsigned)readlane((int)(unsigned)c.mybase, j);
+    const unsigned hi = (unsigned)readlane((int)(unsigned)(c.mybase >> 32), j);
+    return (char*)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ char* out_sf_of(const EpScatterArgs& a, char* rows) {
+    return a.mode == EP_SCATTER_PACK ? rows + a.pack_sf_off : (char*)a.recv_sf;
+}
 
 // A wave task is (row, column part).  Resolves the row's token, its source row and its destination
 // rows; the task of part 0 also writes the row's small items.  Three modes:
@@ -368,27 +480,36 @@ struct RowCtx {
 //                      (partition * max_tokens + slot of dst_buffer_slot_idx); part 0 writes the packed
 //                      metadata [all K topk_idx | all K weights | src_token_global_idx] into each of them
 //                      (impls/ep/dispatch.hpp:768-794, layout/ep/token.hpp:59-82)
-//   EP_SCATTER_REGION  rows of the receive stream, payload, scales and weights read from the packed rows
-//                      of this partition's own region (dispatch_copy_epilogue.hpp:459-522)
+//   EP_SCATTER_REGION  rows of the receive stream (the regions of every source partition in turn), payload,
+//                      scales and weights read from the packed rows; destinations come from the metadata
+//                      rows the receive-side layout wrote (dispatch_copy_epilogue.hpp:459-522)
 __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int i, int part, RowCtx& c) {
     const int lane = lane_id();
     const int K = a.num_topk;
     int myslot = -1, t;
     if (a.mode == EP_SCATTER_PACK) {
+        uint64_t mybase = 0;
         t = i;
         int64_t e = -1;
         if (lane < K) {
             e = a.topk_idx[(int64_t)t * K + lane];
             const int s = a.dst_slot_idx[(int64_t)t * K + lane];
-            if (s >= 0 && s < a.max_tokens && e >= 0 && e < a.num_experts)
-                myslot = (int)(e / a.experts_per_rank) * a.max_tokens + s;
+            if (s >= 0 && s < a.max_tokens && e >= 0 && e < a.num_experts) {
+                const int peer = (int)(e / a.experts_per_rank);
+                myslot = (a.region_by_source ? a.rank_idx : peer) * a.max_tokens + s;
+                mybase = (uint64_t)(a.peer_arenas[peer] + a.buffer_off);
+            }
         }
+        c.t = t;
+        c.myslot = myslot;
+        c.mybase = mybase;
+        c.src_row = t;
         if (part == 0) {
             const float w = (a.topk_weights != nullptr && lane < K) ? a.topk_weights[(int64_t)t * K + lane] : 0.0f;
             for (int j = 0; j < K; ++j) {
                 const int g = readlane(myslot, j);
                 if (g < 0) continue;
-                char* row = (char*)a.recv_x + (int64_t)g * a.out_row_bytes;
+                char* row = out_rows_of(a, c, j) + (int64_t)g * a.out_row_bytes;
                 if (lane < K) {
                     if (a.with_metadata) ((int64_t*)(row + a.idx_off))[lane] = e;
                     ((float*)(row + a.w_off))[lane] = w;
@@ -396,9 +517,18 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
                 if (a.with_metadata && lane == 0) *(int*)(row + a.src_off) = a.rank_idx * a.max_tokens + t;
             }
         }
-        c.t = t;
+        return true;
+    }
+    c.mybase = 0;
+    if (a.mode == EP_SCATTER_REGION) {
+        // the metadata rows are complete before this kernel runs: written by the receive-side layout, or cached
+        const int v = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
+        if (lane < K && v >= 0 && v < a.num_out_rows) myslot = v;
+        c.src_row = region_row_of_stream(a.psum_rank, a.num_ranks, a.max_tokens, i);
+        if (part == 0 && a.recv_topk_weights != nullptr && myslot >= 0)
+            a.recv_topk_weights[myslot] = ((const float*)((const char*)a.x + c.src_row * a.x_row_bytes + a.w_off))[lane];
+        c.t = i;
         c.myslot = myslot;
-        c.src_row = t;
         return true;
     }
     if (!a.cached) {
@@ -419,13 +549,9 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
         if (t < 0 || t >= a.num_tokens) return false;
     }
     if (lane < K && (myslot < 0 || myslot >= a.num_out_rows)) myslot = -1;
-    c.src_row = a.mode == EP_SCATTER_REGION ? a.src_base_row + i : (int64_t)t;
-    if (part == 0 && a.recv_topk_weights != nullptr && lane < K && myslot >= 0) {
-        const float* w = a.mode == EP_SCATTER_REGION
-            ? (const float*)((const char*)a.x + c.src_row * a.x_row_bytes + a.w_off)
-            : a.topk_weights + (int64_t)t * K;
-        a.recv_topk_weights[myslot] = w[lane];
-    }
+    c.src_row = (int64_t)t;
+    if (part == 0 && a.recv_topk_weights != nullptr && lane < K && myslot >= 0)
+        a.recv_topk_weights[myslot] = a.topk_weights[(int64_t)t * K + lane];
     c.t = t;
     c.myslot = myslot;
     return true;
@@ -484,7 +610,7 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
         for (int j = 0; j < K; ++j) {
             const int s = readlane(c.myslot, j);
             if (s < 0) continue;
-            __builtin_nontemporal_store(d, (u32x4*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes) + v);
+            __builtin_nontemporal_store(d, (u32x4*)(out_rows_of(a, c, j) + (int64_t)s * a.out_row_bytes) + v);
         }
     }
     if (part == 0 && a.recv_sf != nullptr) {
@@ -495,7 +621,7 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
             for (int j = 0; j < K; ++j) {
                 const int s = readlane(c.myslot, j);
                 if (s < 0) continue;
-                ((unsigned short*)((char*)a.recv_sf + (int64_t)s * a.out_sf_row_bytes))[p] = val;
+                ((unsigned short*)(out_sf_of(a, out_rows_of(a, c, j)) + (int64_t)s * a.out_sf_row_bytes))[p] = val;
             }
         }
     }
@@ -538,8 +664,9 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     for (int j = 0; j < K; ++j) {
         const int s = readlane(c.myslot, j);
         if (s < 0) continue;
-        __builtin_nontemporal_store(q8, (u32x2*)((char*)a.recv_x + (int64_t)s * a.out_row_bytes) + v);
-        if (writes_scale) ((float*)((char*)a.recv_sf + (int64_t)s * a.out_sf_row_bytes))[v >> 4] = scale;
+        char* rows = out_rows_of(a, c, j);
+        __builtin_nontemporal_store(q8, (u32x2*)(rows + (int64_t)s * a.out_row_bytes) + v);
+        if (writes_scale) ((float*)(out_sf_of(a, rows) + (int64_t)s * a.out_sf_row_bytes))[v >> 4] = scale;
     }
 }
 
@@ -687,7 +814,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
     if (i >= n) return;
 
-    int myslot = -1, t, group = 0;
+    int myslot = -1, t, group = 0, src_rank = 0;
     if (MODE == EP_COMBINE_FINAL) {
         t = i;
         int r = -1;
@@ -704,9 +831,15 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     } else {
         const int mv = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
         if (lane < K && mv >= 0 && mv < a.num_in_rows) myslot = mv;
-        t = readlane(mv, K) - a.rank_idx * a.max_tokens;
-        if (t < 0 || t >= a.max_tokens) return;
-        if (MODE == EP_COMBINE_FUSED && t >= a.num_tokens) return;
+        const int src = readlane(mv, K);                        // source partition * max_tokens + its token
+        if (MODE == EP_COMBINE_PARTIAL) {
+            src_rank = src / a.max_tokens;
+            if (src < 0 || src_rank >= a.num_ranks) return;
+            t = src - src_rank * a.max_tokens;
+        } else {
+            t = src - a.rank_idx * a.max_tokens;
+            if (t < 0 || t >= a.max_tokens || t >= a.num_tokens) return;
+        }
         group = a.num_ranks < K ? a.rank_idx : readlane(mv, K + 1);
         if (MODE == EP_COMBINE_PARTIAL && (group < 0 || group >= a.num_groups)) return;
     }
@@ -714,8 +847,10 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     const int nvec = a.hidden >> 3;
     const int64_t yvec = a.y_row_bytes >> 4;
     const u32x4* y = (const u32x4*)a.y;
-    char* out_row = (char*)a.combined_x +
-        (MODE == EP_COMBINE_PARTIAL ? ((int64_t)group * a.max_tokens + t) : (int64_t)t) * a.out_row_bytes;
+    // a partial goes to the combine buffer of the partition its token came from (impls/ep/combine.hpp:291-324)
+    char* out_row = MODE == EP_COMBINE_PARTIAL
+        ? a.peer_arenas[src_rank] + a.buffer_off + ((int64_t)group * a.max_tokens + t) * a.out_row_bytes
+        : (char*)a.combined_x + (int64_t)t * a.out_row_bytes;
 
     // ---- gate weights ----
     float myw = 0.0f;

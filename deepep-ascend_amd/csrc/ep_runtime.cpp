@@ -197,6 +197,9 @@ struct ep_buffer {
     int seq = 0;                 // sequence number of the last non-cached dispatch
     bool destroyed = false;
     int device = 0;
+    // node of partitions living in this process (ep_buffer_connect): every partition's arena is a peer
+    bool connected = false;
+    std::vector<ep_buffer*> peers;
     // state handed from ep_dispatch_launch to ep_dispatch_epilogue_launch
     struct {
         bool valid = false;
@@ -204,7 +207,15 @@ struct ep_buffer {
         int* slot_map = nullptr;
         int* recv_tok = nullptr;
         bool notified = false;
+        bool recv_done = false;     // more than one partition: the receive-side layout has been enqueued
     } last;
+
+    char* const* peer_table() const { return (char* const*)(arena + EP_WS_PEERS_OFF); }
+    const int* inbox() const { return (const int*)(arena + EP_WS_INBOX_OFF); }
+    // rows the receive stream of this partition can hold
+    int64_t recv_rows_bound(int num_tokens, int max_tokens) const {
+        return connected ? (int64_t)num_ranks * max_tokens : num_tokens;
+    }
 
     char* workspace() const { return arena; }
     char* buffer() const { return arena + kWorkspaceBytes; }
@@ -212,6 +223,28 @@ struct ep_buffer {
 };
 
 namespace {
+// LDS of the layout kernels: histograms / per-wave counters, the staged keys, the per-source row counts
+unsigned layout_key_bytes(int K) { return 2u * EP_TOKENS_PER_BLOCK * K * sizeof(short); }
+unsigned layout_count_lds(int E, int R, int K) {
+    return (unsigned)(E + R + R + EP_LAYOUT_THREADS / 64) * sizeof(int) + layout_key_bytes(K);
+}
+unsigned layout_assign_lds(int E, int R, int K) {
+    const unsigned nw = EP_LAYOUT_THREADS / 64;
+    return (unsigned)(E / R + R + nw * (E + R) + nw + 1 + R + nw) * sizeof(int) + layout_key_bytes(K);
+}
+
+void write_peer_table(ep_buffer* b, const std::vector<char*>& arenas) {
+    std::vector<char*> table(EP_MAX_RANKS, nullptr);
+    for (size_t i = 0; i < arenas.size(); ++i) table[i] = arenas[i];
+    HIP_CHECK(hipMemcpy(b->arena + EP_WS_PEERS_OFF, table.data(), sizeof(char*) * EP_MAX_RANKS, hipMemcpyHostToDevice));
+}
+
+void disconnect(ep_buffer* b) {
+    write_peer_table(b, std::vector<char*>(b->num_ranks, b->arena));
+    b->connected = false;
+    b->peers.clear();
+}
+
 // The code object is loaded on one device and the arena lives there: calls must come with that
 // device current.
 void check_buffer(const ep_buffer* b) {
@@ -322,6 +355,7 @@ int ep_buffer_create(int rank_idx, int num_ranks, int64_t num_bytes, int64_t num
             HIP_CHECK(hipHostMalloc((void**)&b->host_page, EP_HOST_PAGE_INTS * sizeof(int), hipHostMallocMapped));
             memset(b->host_page, 0, EP_HOST_PAGE_INTS * sizeof(int));
             HIP_CHECK(hipHostGetDevicePointer((void**)&b->host_page_dev, b->host_page, 0));
+            write_peer_table(b, std::vector<char*>(num_ranks, b->arena));    // not connected: every peer is this arena
             HIP_CHECK(hipDeviceSynchronize());
         } catch (...) {
             if (b->arena != nullptr) (void)hipFree(b->arena);
@@ -333,11 +367,36 @@ int ep_buffer_create(int rank_idx, int num_ranks, int64_t num_bytes, int64_t num
     });
 }
 
+int ep_buffer_connect(ep_buffer_t** bufs, int n) {
+    return guarded([&] {
+        EP_HOST_ASSERT(bufs != nullptr and n > 1);
+        std::vector<char*> arenas(n);
+        for (int i = 0; i < n; ++i) {
+            check_buffer(bufs[i]);
+            EP_HOST_ASSERT(bufs[i]->num_ranks == n and bufs[i]->rank_idx == i);
+            EP_HOST_ASSERT(bufs[i]->num_buffer_bytes == bufs[0]->num_buffer_bytes);
+            EP_HOST_ASSERT(not bufs[i]->connected);
+            arenas[i] = bufs[i]->arena;
+        }
+        HIP_CHECK(hipDeviceSynchronize());
+        for (int i = 0; i < n; ++i) {
+            write_peer_table(bufs[i], arenas);
+            bufs[i]->connected = true;
+            bufs[i]->peers.assign(bufs, bufs + n);
+        }
+    });
+}
+
 int ep_buffer_destroy(ep_buffer_t* b) {
     return guarded([&] {
         EP_HOST_ASSERT(b != nullptr);
         EP_HOST_ASSERT(not b->destroyed);
         HIP_CHECK(hipDeviceSynchronize());
+        // the other partitions of a node must not keep pointers into this arena
+        const std::vector<ep_buffer*> peers = b->peers;
+        for (ep_buffer* p : peers)
+            if (p != b) disconnect(p);
+        b->peers.clear();
         HIP_CHECK(hipFree(b->arena));
         HIP_CHECK(hipHostFree(b->host_page));
         b->arena = nullptr;
@@ -493,6 +552,13 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             sa.w_off = pk.w_off;
             sa.src_off = pk.src_off;
             sa.num_out_rows = num_ranks * a.num_max_tokens_per_rank;
+            // unconnected: the regions of this arena, one per destination; in a node: region `rank_idx` of
+            // the destination's own arena, where its receive side will look for them
+            sa.peer_arenas = b->peer_table();
+            sa.buffer_off = kWorkspaceBytes;
+            sa.region_by_source = b->connected ? 1 : 0;
+            sa.num_ranks = num_ranks;
+            sa.pack_sf_off = pk.sf_off;
             sa.num_parts = (int)std::max<int64_t>(1, a.fused_fp8_quant ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024));
             sa.num_row_blocks = (int)ceil_div((int64_t)num_tokens * sa.num_parts, EP_ROWS_PER_BLOCK);
             if (sa.num_row_blocks == 0) return;
@@ -511,7 +577,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         const int E = a.num_experts, R = num_ranks, K = num_topk;
         const int num_blocks = std::max<int>(1, (int)ceil_div(num_tokens, EP_TOKENS_PER_BLOCK));
         int* ws = (int*)b->workspace();
-        int64_t off = 0;
+        int64_t off = EP_WS_HEADER_BYTES / sizeof(int);
         auto carve = [&](int64_t n) {
             int* p = ws + off;
             off += align_up(std::max<int64_t>(n, 1), 64);
@@ -522,9 +588,16 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         la.rank_total = carve(R);
         la.blk_expert_cnt = carve((int64_t)num_blocks * E);
         la.blk_rank_cnt = carve((int64_t)num_blocks * R);
-        la.slot_map = carve((int64_t)num_tokens * K);
-        la.recv_tok = carve(a.num_max_tokens_per_rank);
+        if (R == 1) {
+            la.slot_map = carve((int64_t)num_tokens * K);
+            la.recv_tok = carve(a.num_max_tokens_per_rank);
+        }
         EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= kWorkspaceBytes);
+        // more than one partition: this launch is the send side only (slots in the destinations' regions, row
+        // counts into their inboxes); the receive side is ep_dispatch_recv_launch
+        la.send_only = R > 1 ? 1 : 0;
+        la.peer_arenas = b->peer_table();
+        la.connected = b->connected ? 1 : 0;
 
         la.topk_idx = (const int64_t*)a.topk_idx.data;
         la.num_tokens = num_tokens;
@@ -536,8 +609,8 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         la.max_tokens = a.num_max_tokens_per_rank;
         la.experts_per_rank = num_experts_per_rank;
         la.num_blocks = num_blocks;
-        la.seq = ++b->seq;
-        la.notify_host = do_cpu_sync ? 1 : 0;
+        la.seq = R == 1 ? ++b->seq : 0;
+        la.notify_host = do_cpu_sync and R == 1 ? 1 : 0;
         la.dst_buffer_slot_idx = (int*)a.dst_buffer_slot_idx.data;
         la.dst_gsge_idx = (int*)a.dst_gsge_idx.data;
         la.psum_rank = (int*)psum_rank.data;
@@ -546,11 +619,8 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         la.cumulative_stats = (int*)a.cumulative_local_expert_recv_stats.data;
         la.host_page = b->host_page_dev;
 
-        const unsigned key_bytes = 2u * EP_TOKENS_PER_BLOCK * K * sizeof(short);
-        const unsigned smem_count = (unsigned)(E + R) * sizeof(int) + key_bytes;
-        const unsigned nw = EP_LAYOUT_THREADS / 64;
-        const unsigned smem_assign =
-            (unsigned)(num_experts_per_rank + R + nw * (E + R) + nw + 1) * sizeof(int) + key_bytes;
+        const unsigned smem_count = layout_count_lds(E, R, K);
+        const unsigned smem_assign = layout_assign_lds(E, R, K);
         EP_HOST_ASSERT(smem_assign <= 64 * 1024);
         // one block: its own counts are the totals and nothing has to run before the slot assignment
         la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : EP_LAYOUT_SCANNED;
@@ -570,7 +640,96 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         b->last.max_tokens = a.num_max_tokens_per_rank;
         b->last.slot_map = la.slot_map;
         b->last.recv_tok = la.recv_tok;
-        b->last.notified = do_cpu_sync;
+        b->last.notified = do_cpu_sync and R == 1;
+        b->last.recv_done = false;
+    });
+}
+
+int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
+    return guarded([&] {
+        EP_HOST_ASSERT(pa != nullptr);
+        check_buffer(b);
+        const ep_dispatch_recv_args_t& a = *pa;
+        const int R = b->num_ranks;
+        if (R == 1) return;             // one partition: ep_dispatch_launch has produced the whole layout
+        EP_HOST_ASSERT(b->last.valid and not b->last.recv_done and "follows this buffer's own ep_dispatch_launch");
+        const int K = a.num_topk, E = a.num_experts;
+        EP_HOST_ASSERT(K == b->last.num_topk and E == b->last.num_experts);
+        EP_HOST_ASSERT(a.expert_alignment == b->last.alignment and a.num_max_tokens_per_rank == b->last.max_tokens);
+        const int El = E / R;
+        const auto& psum_rank = a.psum_num_recv_tokens_per_rank;
+        const auto& psum_expert = a.psum_num_recv_tokens_per_expert;
+        const auto& unaligned = a.num_unaligned_recv_tokens_per_expert;
+        EP_HOST_ASSERT(present(psum_rank) and psum_rank.ndim == 1 and psum_rank.size[0] == R);
+        EP_HOST_ASSERT(present(psum_expert) and psum_expert.ndim == 1 and psum_expert.size[0] == El);
+        EP_HOST_ASSERT(present(unaligned) and unaligned.ndim == 1 and unaligned.size[0] == El);
+        EP_HOST_ASSERT(psum_rank.dtype == EP_DTYPE_I32 and psum_expert.dtype == EP_DTYPE_I32);
+        EP_HOST_ASSERT(unaligned.dtype == EP_DTYPE_I32);
+        EP_HOST_ASSERT(contiguous(psum_rank) and contiguous(psum_expert) and contiguous(unaligned));
+        if (present(a.cumulative_local_expert_recv_stats)) {
+            const auto& st = a.cumulative_local_expert_recv_stats;
+            EP_HOST_ASSERT(st.ndim == 1 and st.size[0] == El and contiguous(st) and st.dtype == EP_DTYPE_I32);
+        }
+        const auto& meta = a.recv_src_metadata;
+        EP_HOST_ASSERT(present(meta) and meta.ndim == 2 and meta.size[1] == K + 2);
+        EP_HOST_ASSERT(contiguous(meta) and meta.dtype == EP_DTYPE_I32);
+        const int64_t rows_bound = b->recv_rows_bound(b->last.num_tokens, a.num_max_tokens_per_rank);
+        EP_HOST_ASSERT(meta.size[0] >= rows_bound and "room for every row that can arrive");
+        EP_HOST_ASSERT(rows_bound <= INT32_MAX);
+        EP_HOST_ASSERT(a.hidden_bytes > 0 and a.num_sf_packs >= 0);
+        const PackedToken pk = packed_token(a.hidden_bytes, a.num_sf_packs * 2, K, true);
+        EP_HOST_ASSERT((int64_t)R * a.num_max_tokens_per_rank * pk.bytes <= b->num_buffer_bytes);
+
+        const int num_blocks = std::max<int>(1, (int)ceil_div(rows_bound, EP_TOKENS_PER_BLOCK));
+        int* ws = (int*)b->workspace();
+        int64_t off = EP_WS_HEADER_BYTES / sizeof(int);
+        auto carve = [&](int64_t n) {
+            int* p = ws + off;
+            off += align_up(std::max<int64_t>(n, 1), 64);
+            return p;
+        };
+        EpLayoutArgs la{};
+        la.expert_total = carve(E);
+        la.rank_total = carve(R);
+        la.blk_expert_cnt = carve((int64_t)num_blocks * E);
+        la.blk_rank_cnt = carve((int64_t)num_blocks * R);
+        EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= kWorkspaceBytes and "layout scratch of the receive stream fits the workspace");
+        la.recv_mode = 1;
+        la.num_tokens = (int)rows_bound;
+        la.num_topk = K;
+        la.num_experts = E;
+        la.num_ranks = R;
+        la.rank_idx = b->rank_idx;
+        la.expert_alignment = a.expert_alignment;
+        la.max_tokens = a.num_max_tokens_per_rank;
+        la.experts_per_rank = El;
+        la.num_blocks = num_blocks;
+        la.seq = ++b->seq;
+        la.notify_host = a.do_cpu_sync ? 1 : 0;
+        la.psum_rank = (int*)psum_rank.data;
+        la.psum_expert = (int*)psum_expert.data;
+        la.unaligned_expert = (int*)unaligned.data;
+        la.cumulative_stats = (int*)a.cumulative_local_expert_recv_stats.data;
+        la.host_page = b->host_page_dev;
+        la.peer_arenas = b->peer_table();
+        la.connected = b->connected ? 1 : 0;
+        la.inbox = b->inbox();
+        la.packed_base = b->buffer();
+        la.packed_row_bytes = pk.bytes;
+        la.idx_off = pk.idx_off;
+        la.src_off = pk.src_off;
+        la.recv_src_metadata = (int*)meta.data;
+        la.rows_cap = (int)std::min<int64_t>(meta.size[0], INT32_MAX);
+        la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : EP_LAYOUT_SCANNED;
+        const unsigned smem_assign = layout_assign_lds(E, R, K);
+        EP_HOST_ASSERT(smem_assign <= 64 * 1024);
+        if (la.scan_mode == EP_LAYOUT_SCANNED) {
+            launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, layout_count_lds(E, R, K), a.stream, la);
+            launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 64), EP_SCAN_THREADS, 0, a.stream, la);
+        }
+        launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, a.stream, la);
+        b->last.recv_done = true;
+        b->last.notified = a.do_cpu_sync != 0;
     });
 }
 
@@ -664,6 +823,7 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         if (not cached_mode) {
             EP_HOST_ASSERT(b->last.valid and "the copy epilogue follows its own dispatch launch");
             EP_HOST_ASSERT(b->last.num_tokens == num_tokens and b->last.num_topk == K);
+            EP_HOST_ASSERT((R == 1 or b->last.recv_done) and "the receive-side layout comes before the copy");
         }
 
         EpScatterArgs sa{};
@@ -682,7 +842,8 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.hidden = hidden;
         sa.num_topk = K;
         // never walk past the rows the metadata tensor holds
-        sa.num_rows_bound = (int)std::min<int64_t>(num_tokens, a.recv_src_metadata.size[0]);
+        sa.num_rows_bound = (int)std::min<int64_t>(b->recv_rows_bound(num_tokens, a.num_max_tokens_per_rank),
+                                                   a.recv_src_metadata.size[0]);
         sa.num_tokens = num_tokens;
         sa.rank_idx = b->rank_idx;
         sa.max_tokens = a.num_max_tokens_per_rank;
@@ -711,10 +872,11 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
             const PackedToken pk = packed_token(hidden * payload_elem, sf_packs * 2, K, not cached_mode);
             EP_HOST_ASSERT((int64_t)R * a.num_max_tokens_per_rank * pk.bytes <= b->num_buffer_bytes);
             sa.mode = EP_SCATTER_REGION;
+            sa.psum_rank = (const int*)a.psum_num_recv_tokens_per_rank.data;
+            sa.num_ranks = R;
             sa.x = b->buffer();
             sa.x_row_bytes = pk.bytes;
             sa.copy_bytes = (int64_t)hidden * payload_elem;
-            sa.src_base_row = (int64_t)b->rank_idx * a.num_max_tokens_per_rank;
             sa.sf = sf_packs > 0 ? b->buffer() + pk.sf_off : nullptr;
             sa.sf_token_stride_bytes = pk.bytes;
             sa.sf_pack_stride_bytes = 2;
@@ -828,6 +990,8 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             ca.num_recv_ptr = (const int*)psum_rank.data + (R - 1);
             ca.num_rows_bound = (int)a.src_metadata.size[0];
             ca.combined_x = b->buffer();
+            ca.peer_arenas = b->peer_table();
+            ca.buffer_off = kWorkspaceBytes;
             ca.out_row_bytes = combine_token;
             ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
             if (ca.num_row_blocks == 0) return;

@@ -49,6 +49,16 @@ class _DispatchEpilogueArgs(ctypes.Structure):
         ('fused_fp8_quant', ctypes.c_int32), ('recv_sf_layout', ctypes.c_int32), ('stream', ctypes.c_void_p)]
 
 
+class _DispatchRecvArgs(ctypes.Structure):
+    _fields_ = [(n, _Tensor) for n in (
+        'psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert', 'num_unaligned_recv_tokens_per_expert',
+        'cumulative_local_expert_recv_stats', 'recv_src_metadata')] + [
+        ('hidden_bytes', ctypes.c_int32), ('num_sf_packs', ctypes.c_int32), ('num_topk', ctypes.c_int32),
+        ('num_max_tokens_per_rank', ctypes.c_int32), ('num_experts', ctypes.c_int32),
+        ('expert_alignment', ctypes.c_int32), ('do_cpu_sync', ctypes.c_int32), ('reserved', ctypes.c_int32),
+        ('stream', ctypes.c_void_p)]
+
+
 class _CombineArgs(ctypes.Structure):
     _fields_ = [(n, _Tensor) for n in (
         'x', 'topk_weights', 'bias_0', 'bias_1', 'src_metadata', 'combined_topk_idx',
@@ -87,6 +97,8 @@ _ep_dispatch = _sig('ep_dispatch_launch', ctypes.c_int, ctypes.c_void_p, ctypes.
 _ep_wait = _sig('ep_dispatch_wait_counts', ctypes.c_int, ctypes.c_void_p, _c_int_p, _c_int_p, _c_int_p)
 _ep_worst = _sig('ep_dispatch_worst_case_sizes', ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                  ctypes.c_int, ctypes.c_int, _c_int_p, _c_int_p)
+_ep_dispatch_recv = _sig('ep_dispatch_recv_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_DispatchRecvArgs))
+_ep_connect = _sig('ep_buffer_connect', ctypes.c_int, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int)
 _ep_dispatch_epi = _sig('ep_dispatch_epilogue_launch', ctypes.c_int, ctypes.c_void_p,
                         ctypes.POINTER(_DispatchEpilogueArgs))
 _ep_combine = _sig('ep_combine_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_CombineArgs), ctypes.c_int)
@@ -277,6 +289,7 @@ class EPBuffer(BufferBase):
         _check(_ep_create(rank_idx, num_ranks, num_bytes, num_lb_bytes, num_cpu_timeout_secs, num_gpu_timeout_secs,
                           ctypes.byref(handle)))
         self._h = handle
+        self.connected = False
         self.device = torch.device('cuda', torch.cuda.current_device())
         self.context = Context(rank_idx, num_ranks)
         self.main_context = self.context
@@ -310,6 +323,15 @@ class EPBuffer(BufferBase):
 
     def print_memory_usage(self) -> None:
         _check(_ep_print_mem(self._h))
+
+    @staticmethod
+    def connect(runtimes) -> None:
+        """Makes the given runtime objects (partition i of n at index i) one node: packed rows, row counts
+        and combine partials then go straight into the arena of the partition they are meant for."""
+        handles = (ctypes.c_void_p * len(runtimes))(*[r._h for r in runtimes])
+        _check(_ep_connect(handles, len(runtimes)))
+        for r in runtimes:
+            r.connected = True
 
     def region(self, which: int) -> Tuple[int, int]:
         n = ctypes.c_int64()
@@ -390,10 +412,45 @@ class EPBuffer(BufferBase):
             # the descriptors hold raw pointers: the inputs stay referenced until the copy kernel is enqueued
             assert keep_alive is not None
             per_expert_list: List[int] = []
+            partitioned = self.num_ranks > 1
+            # rows that can arrive: this partition's own tokens, or everybody's when the partitions form a node
+            rows_bound = self.num_ranks * num_max_tokens_per_rank if self.connected else num_tokens
+            recv_src_metadata = None
+            if partitioned and not cached_mode:
+                # receive side: count and rank the rows that arrived in this partition's regions
+                c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
+                _check(_ep_worst(self._h, num_max_tokens_per_rank, num_topk, num_experts, expert_alignment,
+                                 ctypes.byref(c_recv), ctypes.byref(c_exp)))
+                recv_src_metadata = ints(rows_bound if do_cpu_sync else c_recv.value, num_topk + 2)
+                r = _DispatchRecvArgs()
+                r.psum_num_recv_tokens_per_rank, r.psum_num_recv_tokens_per_expert = a.psum_num_recv_tokens_per_rank, \
+                    a.psum_num_recv_tokens_per_expert
+                r.num_unaligned_recv_tokens_per_expert = a.num_unaligned_recv_tokens_per_expert
+                r.cumulative_local_expert_recv_stats = a.cumulative_local_expert_recv_stats
+                r.recv_src_metadata = _desc(recv_src_metadata)
+                r.hidden_bytes = hidden * (1 if fused_fp8_quant else x.element_size())
+                r.num_sf_packs = 2 * ((hidden + 127) // 128) if fused_fp8_quant else (sf.size(1) if sf is not None else 0)
+                r.num_topk, r.num_max_tokens_per_rank = num_topk, num_max_tokens_per_rank
+                r.num_experts, r.expert_alignment = num_experts, expert_alignment
+                r.do_cpu_sync = int(do_cpu_sync)
+                r.stream = _stream()
+                _check(_ep_dispatch_recv(self._h, ctypes.byref(r)))
+
+            def wait_counts():
+                c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
+                c_list = (ctypes.c_int * max(1, num_local_experts))()
+                _check(_ep_wait(self._h, ctypes.byref(c_recv), ctypes.byref(c_exp), c_list))
+                return c_recv.value, c_exp.value, [c_list[i] for i in range(num_local_experts)]
+
             if cached_mode:
                 num_recv, num_expanded = cached_num_recv_tokens, cached_num_expanded_tokens
                 per_expert_list = cached_num_recv_tokens_per_expert_list
                 alloc_recv, alloc_expanded = num_recv, num_expanded
+            elif do_cpu_sync and self.connected:
+                # a node: the bound over every partition's tokens is far above what arrives; wait for the counts
+                num_recv, num_expanded, per_expert_list = wait_counts()
+                alloc_recv, alloc_expanded = num_recv, num_expanded
+                recv_src_metadata = recv_src_metadata[:num_recv]
             elif do_cpu_sync:
                 # Exact sizes come from the host count page, but waiting for it here would leave the GPU
                 # idle between the layout kernels and the copy.  Allocate for this call's upper bound,
@@ -430,7 +487,7 @@ class EPBuffer(BufferBase):
                 recv_src_metadata = cached_recv_src_metadata
                 if recv_src_metadata.dim() != 2 or recv_src_metadata.size(0) != num_recv:
                     raise EPException('Assertion exception (_C.py): recv_src_metadata.size(0) == num_recv_tokens')
-            else:
+            elif recv_src_metadata is None:
                 recv_src_metadata = ints(alloc_recv, num_topk + 2)
 
             e = _DispatchEpilogueArgs()
@@ -451,11 +508,7 @@ class EPBuffer(BufferBase):
             _check(_ep_dispatch_epi(self._h, ctypes.byref(e)))
 
             if num_recv is None:
-                c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
-                c_list = (ctypes.c_int * max(1, num_local_experts))()
-                _check(_ep_wait(self._h, ctypes.byref(c_recv), ctypes.byref(c_exp), c_list))
-                num_recv, num_expanded = c_recv.value, c_exp.value
-                per_expert_list = [c_list[i] for i in range(num_local_experts)]
+                num_recv, num_expanded, per_expert_list = wait_counts()
                 if num_recv > alloc_recv or num_expanded > alloc_expanded:
                     raise EPException('Assertion exception (_C.py): received counts exceed this call\'s bound')
                 recv_x = recv_x[:num_expanded]

@@ -6,7 +6,7 @@ from ._C import init_jit as _init_jit
 _init_jit()
 
 from . import comm                                                                   # noqa: E402
-from .comm import (LocalGroup, destroy_all_managed_hccl_comm, get_logical_domain_size,   # noqa: E402
+from .comm import (LocalGroup, LocalNode, destroy_all_managed_hccl_comm, get_logical_domain_size,   # noqa: E402
                    get_physical_domain_size)
 from .buffers.allocator import BufferAllocator                                       # noqa: E402
 from .buffers.base import BufferBase                                                 # noqa: E402

@@ -150,6 +150,9 @@ class EPBuffer(BufferBase):
                                    num_lb_bytes, use_huge1g_page, num_cpu_timeout_secs, num_gpu_timeout_secs,
                                    explicitly_destroy)
         self.context = self.runtime.context
+        node = getattr(group, 'node', None)
+        if node is not None:
+            node.register(self.rank_idx, self.runtime)      # the last partition of a node connects them all
         if plan is not None:
             plan.materialize(self.runtime.lb_storage)
         self.num_scaleout_ranks, self.num_scaleup_ranks = self.get_logical_domain_size()

@@ -9,15 +9,42 @@ class LocalGroup:
     """Duck-typed process group (`rank()`, `size()`) describing one of `size` virtual partitions
     that live on this GPU; lets `EPBuffer` run one GPU's share of an EP-`size` layout."""
 
-    def __init__(self, rank: int = 0, size: int = 1, name: str = 'local'):
+    def __init__(self, rank: int = 0, size: int = 1, name: str = 'local', node: Optional['LocalNode'] = None):
         assert 0 <= rank < size
-        self._rank, self._size, self.name = rank, size, name
+        self._rank, self._size, self.name, self.node = rank, size, name, node
 
     def rank(self) -> int:
         return self._rank
 
     def size(self) -> int:
         return self._size
+
+
+class LocalNode:
+    """All `size` partitions of an EP group in this process, on this GPU.  Build one `EPBuffer` per
+    `node.group(rank)`; once the last one exists they are connected: a dispatch of partition s stores
+    its packed rows straight into partition r's arena and a combine stores its partials into the arena
+    of the partition the token came from, as ranks do through symmetric memory in the reference.
+    Nothing waits across partitions, so drive them phase by phase on one stream, which the deferred
+    epilogues of the reference API allow:
+
+        events = [buf[r].dispatch(x[r], ..., async_with_compute_stream=True, defer_epilogue=True) for r in ranks]
+        results = [ev.current_stream_wait() for ev in events]      # receive side of every partition
+    and the same for combine."""
+
+    def __init__(self, size: int, name: str = 'node'):
+        assert size > 1
+        self.size, self.name = size, name
+        self._groups = [LocalGroup(r, size, f'{name}{r}', node=self) for r in range(size)]
+        self._runtimes = [None] * size
+
+    def group(self, rank: int) -> LocalGroup:
+        return self._groups[rank]
+
+    def register(self, rank: int, runtime: Any) -> None:
+        self._runtimes[rank] = runtime
+        if all(r is not None for r in self._runtimes):
+            type(runtime).connect(self._runtimes)
 
 
 class LocalCommHandle:

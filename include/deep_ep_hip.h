@@ -83,6 +83,19 @@ void ep_set_fp8_hw_convert(int enable);
  * csrc/kernels/comm/api.hpp:34-64, csrc/kernels/comm/symmetric.hpp:11-29). */
 int ep_buffer_create(int rank_idx, int num_ranks, int64_t num_bytes, int64_t num_lb_bytes,
                      int num_cpu_timeout_secs, int num_gpu_timeout_secs, ep_buffer_t** out);
+/* Makes bufs[0..n) the n partitions of one node living in this process: bufs[i] must be partition i
+ * of n, all on the current device with equal buffer sizes.  From then on a dispatch of partition s
+ * stores the packed rows for partition r straight into region s of r's arena and leaves the row
+ * count in r's inbox, and the owner-side combine stores each partial into the arena of the
+ * partition its token came from: what the reference does through symmetric memory
+ * (csrc/kernels/comm/symmetric.hpp:11-29, impls/ep/dispatch.hpp:768-794, impls/ep/combine.hpp:291-324),
+ * with plain device pointers standing where peer-mapped ones would on several GPUs.  There are no
+ * cross-partition waits: the caller orders the launches (every partition's ep_dispatch_launch
+ * before any ep_dispatch_recv_launch; every copy epilogue before any combine; every combine phase 0
+ * before any phase 1), e.g. by enqueueing them in that order on one stream.  Destroying a
+ * partition disconnects the others.  Synchronises.  No counterpart call in the reference, whose
+ * ranks find each other through the process group. */
+int ep_buffer_connect(ep_buffer_t** bufs, int n);
 /* EPBuffer::destroy (csrc/buffers/ep.hpp:65-73). */
 int ep_buffer_destroy(ep_buffer_t* buf);
 /* which: 0 workspace, 1 buffer, 2 lb storage (csrc/buffers/ep.hpp:50-53). */
@@ -110,8 +123,34 @@ typedef struct ep_dispatch_args {
 } ep_dispatch_args_t;
 
 /* Validates like EPBuffer::dispatch (csrc/buffers/ep.hpp:113-246) and enqueues the layout
- * kernels: replaces launch_dispatch (csrc/kernels/ep/dispatch.hpp:20-82). */
+ * kernels: replaces launch_dispatch (csrc/kernels/ep/dispatch.hpp:20-82).  With more than one
+ * partition this is the send side (dst_buffer_slot_idx, dst_gsge_idx, packed rows, inbox counts)
+ * and ep_dispatch_recv_launch writes the other handle tensors. */
 int ep_dispatch_launch(ep_buffer_t* buf, const ep_dispatch_args_t* args);
+
+typedef struct ep_dispatch_recv_args {
+    /* handle tensors, written here (csrc/buffers/ep.hpp:205-246) */
+    ep_tensor_t psum_num_recv_tokens_per_rank;          /* [R] int32 */
+    ep_tensor_t psum_num_recv_tokens_per_expert;        /* [E/R] int32 */
+    ep_tensor_t num_unaligned_recv_tokens_per_expert;   /* [E/R] int32 */
+    ep_tensor_t cumulative_local_expert_recv_stats;     /* [E/R] int32 (optional) */
+    ep_tensor_t recv_src_metadata;                      /* [>= rows that can arrive, K+2] int32 out */
+    int32_t hidden_bytes, num_sf_packs;                 /* payload bytes and 2-byte scale packs of a packed row */
+    int32_t num_topk, num_max_tokens_per_rank, num_experts, expert_alignment;
+    int32_t do_cpu_sync, reserved;
+    void* stream;
+} ep_dispatch_recv_args_t;
+
+/* More than one partition, non-cached dispatch: the receive side of launch_dispatch and the slot
+ * assignment of the copy epilogue (impls/ep/dispatch.hpp:469-545,
+ * impls/ep/dispatch_copy_epilogue.hpp:130-174,397-423,471-488,514-522).  Walks the rows that
+ * arrived in this partition's regions (source partitions in turn, each up to its inbox count),
+ * ranks them per local expert and writes the handle tensors, the metadata rows and, with
+ * do_cpu_sync, the host counts.  Rows can arrive from n * num_max_tokens_per_rank tokens in a
+ * node, from the dispatched tokens otherwise.  A no-op with one partition.  Call it after
+ * ep_dispatch_launch (of every partition of a node) and before ep_dispatch_wait_counts /
+ * ep_dispatch_epilogue_launch. */
+int ep_dispatch_recv_launch(ep_buffer_t* buf, const ep_dispatch_recv_args_t* args);
 
 /* Host wait for the counts of the last non-cached do_cpu_sync dispatch, with the buffer's CPU
  * timeout ("reduction timeout").  per_expert receives E/R aligned counts.  Replaces the

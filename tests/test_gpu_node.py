@@ -1,0 +1,241 @@
+"""Every partition of an EP group on this one GPU, connected into a node: the dispatch of partition s
+puts its packed rows and row counts straight into the arena of the partition they are for, the
+receive side of each partition lays out whatever arrived, and the combine sends every partial back
+to the arena its token came from.  Driven phase by phase through the deferred epilogues of the
+reference API, on one stream.  Checked against the multi-rank oracle and against the vectors the
+reference's own refs.dispatch / refs.combine produced under 2- and 4-rank gloo groups.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_bits, make_routing, make_tokens
+from oracle import ep_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden')
+
+
+def make_node(R, max_tokens, H, K, fp8):
+    import deep_ep
+    node = deep_ep.LocalNode(R)
+    return [deep_ep.EPBuffer(node.group(r), num_max_tokens_per_rank=max_tokens, hidden=H, num_topk=K,
+                             use_fp8_dispatch=fp8, explicitly_destroy=True) for r in range(R)]
+
+
+def dispatch_all(bufs, xs, topks, ws, **kw):
+    events = [b.dispatch(x, topk_idx=t, topk_weights=w, async_with_compute_stream=True, defer_epilogue=True, **kw)
+              for b, x, t, w in zip(bufs, xs, topks, ws)]                  # send side of every partition
+    return [ev.current_stream_wait() for ev in events]                    # then every receive side
+
+
+def combine_all(bufs, ys, handles, weights, biases):
+    events = [b.combine(y, h, topk_weights=w, bias=bias, async_with_compute_stream=True, defer_epilogue=True)
+              for b, y, h, w, bias in zip(bufs, ys, handles, weights, biases)]   # owner-side partials everywhere
+    return [ev.current_stream_wait() for ev in events]                           # then the token-side reduces
+
+
+def oracle_dispatch(rows, sfs, topks, ws, E, R, A, max_tokens):
+    """Per destination: the received stream parsed back into its parts, and its layout."""
+    K = topks[0].shape[1]
+    HB = rows[0].shape[1]
+    SB = 0 if sfs[0] is None else sfs[0].shape[1]
+    tok = O.dispatch_token_layout(HB, SB // 2, K)
+    sends = [O.send_layout(t, E, R) for t in topks]
+    regions = [O.pack_regions(rows[s], sfs[s], topks[s], ws[s], sends[s][0], sends[s][1], E, R, s, max_tokens)
+               for s in range(R)]
+    out = []
+    for d in range(R):
+        stream = np.concatenate([regions[s][d] for s in range(R)], axis=0)
+        counts = [regions[s][d].shape[0] for s in range(R)]
+        idx = stream[:, tok.topk_idx_offset:tok.topk_idx_offset + 8 * K].copy().view(np.int64)
+        w = stream[:, tok.topk_weights_offset:tok.topk_weights_offset + 4 * K].copy().view(np.float32)
+        src = stream[:, tok.src_token_global_idx_offset:tok.src_token_global_idx_offset + 4].copy().view(np.int32)[:, 0]
+        lay = O.recv_layout(idx, src, counts, E, R, d, A)
+        hid = stream[:, :HB]
+        sf = stream[:, tok.sf_offset:tok.sf_offset + SB] if SB else None
+        ex, es, ew = O.expand(hid, sf, w, lay['recv_src_metadata'], lay['num_expanded_tokens'])
+        out.append(dict(lay=lay, x=ex, sf=es, w=ew, stream=stream, counts=counts))
+    return sends, out
+
+
+NODE_CASES = [
+    # R, max_tokens, H, E, K, A, masked
+    (2, 96, 256, 8, 3, 1, 0.0),
+    (4, 150, 512, 32, 6, 16, 0.15),        # R < K: partial groups are partitions
+    (8, 70, 256, 64, 4, 128, 0.2),         # R >= K: partial groups are top-k positions
+    (3, 260, 384, 12, 5, 8, 0.3),          # receive streams longer than one layout block
+]
+
+
+@pytest.mark.parametrize('R,max_tokens,H,E,K,A,masked', NODE_CASES)
+@pytest.mark.parametrize('mode', ['bf16', 'fp8_fused', 'fp8_prequant'])
+@pytest.mark.parametrize('do_cpu_sync', [True, False])
+def test_node_dispatch_combine(R, max_tokens, H, E, K, A, masked, mode, do_cpu_sync):
+    if not do_cpu_sync and mode == 'fp8_prequant':
+        pytest.skip('the host sync does not interact with the input format')
+    bufs = make_node(R, max_tokens, H, K, mode != 'bf16')
+    Ts = [max(1, max_tokens - 7 * r) for r in range(R)]                   # ragged token counts
+    xs = [make_tokens(T, H, seed=10 * R + r, outliers=True) for r, T in enumerate(Ts)]
+    routing = [make_routing(T, E, K, seed=20 * R + r, masked=masked) for r, T in enumerate(Ts)]
+    topks, ws = [t for t, _ in routing], [w for _, w in routing]
+    quant = [O.quantise(x) for x in xs]
+    if mode == 'bf16':
+        rows = [bf16_bits(x).view(np.uint8).reshape(x.size(0), -1) for x in xs]
+        sfs = [None] * R
+        gx = [x.to(DEV) for x in xs]
+    else:
+        rows = [q.numpy() for q, _ in quant]
+        sfs = [s.numpy().view(np.uint8).reshape(s.size(0), -1) for _, s in quant]
+        gx = [x.to(DEV) for x in xs] if mode == 'fp8_fused' else \
+            [(q.view(torch.float8_e4m3fn).to(DEV), s.view(torch.int16).to(DEV)) for q, s in quant]
+    sends, want = oracle_dispatch(rows, sfs, [t.numpy() for t in topks], [w.numpy() for w in ws], E, R, A, max_tokens)
+
+    stats = [torch.zeros(E // R, dtype=torch.int32, device=DEV) for _ in range(R)]
+    events = [bufs[r].dispatch(gx[r], topk_idx=topks[r].to(DEV), topk_weights=ws[r].to(DEV),
+                               cumulative_local_expert_recv_stats=stats[r], num_experts=E,
+                               num_max_tokens_per_rank=max_tokens, expert_alignment=A, do_expand=True,
+                               do_zero_padding=True, do_cpu_sync=do_cpu_sync, async_with_compute_stream=True,
+                               defer_epilogue=True, fused_fp8_quant=mode == 'fp8_fused') for r in range(R)]
+    outs = [ev.current_stream_wait() for ev in events]
+    torch.cuda.synchronize()
+
+    handles = []
+    for r, (recv, _, rw, handle) in enumerate(outs):
+        lay = want[r]['lay']
+        n, ne = lay['num_recv_tokens'], lay['num_expanded_tokens']
+        assert np.array_equal(handle.dst_buffer_slot_idx.cpu().numpy(), sends[r][0])
+        assert np.array_equal(handle.psum_num_recv_tokens_per_rank.cpu().numpy(), lay['psum_num_recv_tokens_per_rank'])
+        assert np.array_equal(handle.psum_num_recv_tokens_per_expert.cpu().numpy(), lay['psum_num_recv_tokens_per_expert'])
+        assert np.array_equal(handle.num_unaligned_recv_tokens_per_expert.cpu().numpy(),
+                              lay['num_unaligned_recv_tokens_per_expert'])
+        assert np.array_equal(stats[r].cpu().numpy(), lay['num_unaligned_recv_tokens_per_expert'])
+        assert np.array_equal(handle.recv_src_metadata.cpu().numpy()[:n], lay['recv_src_metadata'])
+        if do_cpu_sync:
+            assert handle.num_recv_tokens == n and handle.num_expanded_tokens == ne
+            assert handle.num_recv_tokens_per_expert_list == lay['num_recv_tokens_per_expert_list']
+            assert handle.recv_src_metadata.size(0) == n
+        else:
+            assert (handle.num_recv_tokens, handle.num_expanded_tokens) == O.no_sync_sizes(R, max_tokens, K, E, A)
+        rx, rsf = recv if isinstance(recv, tuple) else (recv, None)
+        assert np.array_equal(rx.view(torch.uint8).cpu().numpy().reshape(rx.size(0), -1)[:ne], want[r]['x'])
+        if rsf is not None:
+            assert np.array_equal(rsf.contiguous().view(torch.uint8).cpu().numpy().reshape(rsf.size(0), -1)[:ne],
+                                  want[r]['sf'])
+        assert np.array_equal(rw.cpu().numpy().view(np.uint32)[:ne], want[r]['w'].view(np.uint32))
+        handles.append(handle)
+
+    # combine: every owner reduces what it received and sends the partial home
+    g = torch.Generator().manual_seed(R)
+    ys = [torch.randn((outs[r][0][0].size(0) if isinstance(outs[r][0], tuple) else outs[r][0].size(0), H),
+                      generator=g).to(torch.bfloat16) for r in range(R)]
+    for nbias in (0, 2):
+        biases = [[torch.randn((Ts[r], H), generator=g).to(torch.bfloat16) for _ in range(nbias)] for r in range(R)]
+        cevs = [bufs[r].combine(ys[r].to(DEV), handles[r], topk_weights=outs[r][2],
+                                bias=tuple(b.to(DEV) for b in biases[r]) if nbias else None,
+                                async_with_compute_stream=True, defer_epilogue=True) for r in range(R)]
+        res = [ev.current_stream_wait() for ev in cevs]
+        torch.cuda.synchronize()
+        parts, wvecs = {}, {}
+        for r in range(R):
+            lay = want[r]['lay']
+            p, wv = O.combine_partial(ys[r], torch.from_numpy(want[r]['w']), lay['recv_src_metadata'], R, r, max_tokens)
+            assert not set(p) & set(parts)
+            parts.update(p)
+            wvecs.update(wv)
+        for s in range(R):
+            ox, ow = O.combine_final(topks[s].numpy(), E, R, s, max_tokens, lambda k: parts[k], lambda k: wvecs[k],
+                                     biases[s][0] if nbias else None, biases[s][1] if nbias else None, H, True)
+            cx, cw = res[s]
+            assert np.array_equal(bf16_bits(cx), bf16_bits(ox)), (nbias, s)
+            assert torch.equal(cw.cpu(), ow) and torch.equal(cw.cpu(), ws[s])
+    for b in bufs:
+        b.destroy()
+
+
+def test_node_reproduces_the_reference_dispatch_vectors():
+    """tests/golden/dispatch_golden_w2.npz: inputs of both ranks and what refs.dispatch gave each of them
+    (received rows in source order, local expert ids, weights, source tokens, per-source counts)."""
+    g = np.load(os.path.join(GOLD, 'dispatch_golden_w2.npz'))
+    R = 2
+    T0, K, E, H, max_tokens, world = g['r0.cfg'].tolist()
+    assert world == R
+    bufs = make_node(R, max_tokens, H, K, False)
+    xs = [torch.from_numpy(g[f'r{r}.x'].view(np.int16)).view(torch.bfloat16) for r in range(R)]
+    topks = [torch.from_numpy(g[f'r{r}.topk_idx']) for r in range(R)]
+    ws = [torch.from_numpy(g[f'r{r}.topk_weights']) for r in range(R)]
+    outs = dispatch_all(bufs, [x.to(DEV) for x in xs], [t.to(DEV) for t in topks], [w.to(DEV) for w in ws],
+                        num_experts=E, num_max_tokens_per_rank=max_tokens, expert_alignment=4, do_expand=True,
+                        do_zero_padding=True)
+    torch.cuda.synchronize()
+    epr = E // R
+    for d, (rx, _, rw, handle) in enumerate(outs):
+        counts = g[f'r{d}.num_recv_tokens_per_rank']
+        assert np.array_equal(handle.psum_num_recv_tokens_per_rank.cpu().numpy(), np.cumsum(counts))
+        meta = handle.recv_src_metadata.cpu().numpy()
+        assert np.array_equal(meta[:, K], g[f'r{d}.recv_src_token_idx'])
+        want_idx = g[f'r{d}.recv_topk_idx']                      # local expert id or -1
+        assert np.array_equal(meta[:, :K] >= 0, want_idx >= 0)
+        psum = np.concatenate([[0], handle.psum_num_recv_tokens_per_expert.cpu().numpy()])
+        got_x, got_w = bf16_bits(rx), rw.cpu().numpy()
+        for i in range(meta.shape[0]):
+            for j in range(K):
+                s = meta[i, j]
+                if s < 0:
+                    continue
+                e = want_idx[i, j]
+                assert (psum[e] + 3) // 4 * 4 <= s < psum[e + 1]        # inside the expert's aligned block
+                assert np.array_equal(got_x[s], g[f'r{d}.recv_x'][i])
+                assert got_w[s] == g[f'r{d}.recv_topk_weights'][i, j]
+        for e in range(epr):
+            assert psum[e + 1] - (psum[e] + 3) // 4 * 4 == int((want_idx == e).sum())
+    for b in bufs:
+        b.destroy()
+
+
+@pytest.mark.parametrize('world', [2, 4])
+def test_node_reproduces_the_reference_combine_vectors(world):
+    """tests/golden/combine_golden_w{2,4}.npz: expert outputs per (token, selection) of rank 0's tokens and
+    what refs.combine(reduce_in_local=True) made of them."""
+    g = np.load(os.path.join(GOLD, f'combine_golden_w{world}.npz'))
+    for ci in range(5):
+        p = f'w{world}.c{ci}.'
+        T, K, E, H, nbias, W = g[p + 'cfg'].tolist()
+        assert W == world
+        bufs = make_node(W, T, H, K, False)
+        topk = torch.from_numpy(g[p + 'topk_idx'])
+        y3 = torch.from_numpy(g[p + 'y'].view(np.int16)).view(torch.bfloat16)          # [T, K, H]
+        bias = [torch.from_numpy(g[p + f'bias{b}'].view(np.int16)).view(torch.bfloat16) for b in range(nbias)]
+        # rank 0 owns the tokens; the other ranks dispatch a single token that selects nothing
+        xs = [torch.zeros((T if r == 0 else 1, H), dtype=torch.bfloat16) for r in range(W)]
+        topks = [topk if r == 0 else torch.full((1, K), -1, dtype=torch.int64) for r in range(W)]
+        ws = [torch.zeros(t.shape, dtype=torch.float32) for t in topks]
+        outs = dispatch_all(bufs, [x.to(DEV) for x in xs], [t.to(DEV) for t in topks], [w.to(DEV) for w in ws],
+                            num_experts=E, num_max_tokens_per_rank=T, expert_alignment=2, do_expand=True,
+                            do_zero_padding=True)
+        torch.cuda.synchronize()
+        ys = []
+        for r, (rx, _, _, handle) in enumerate(outs):
+            meta = handle.recv_src_metadata.cpu().numpy()
+            y = torch.full((rx.size(0), H), 7.0, dtype=torch.bfloat16)              # padding rows hold garbage
+            for i in range(meta.shape[0]):
+                for j in range(K):
+                    if meta[i, j] >= 0:
+                        y[meta[i, j]] = y3[meta[i, K], j]
+            ys.append(y.to(DEV))
+        handles = [o[3] for o in outs]
+        biases = [(tuple(b.to(DEV) for b in bias) if nbias == 2 else bias[0].to(DEV)) if (r == 0 and nbias) else
+                  (None if nbias == 0 else (tuple(torch.zeros((1, H), dtype=torch.bfloat16, device=DEV) for _ in range(2))
+                                            if nbias == 2 else torch.zeros((1, H), dtype=torch.bfloat16, device=DEV)))
+                  for r in range(W)]
+        res = combine_all(bufs, ys, handles, [None] * W, biases)
+        torch.cuda.synchronize()
+        got, want = bf16_bits(res[0][0]), g[p + 'out']
+        # the reference zeroes masked selections and adds exact zeros: only the sign of a zero may differ
+        same = (got == want) | (((got | want) & 0x7fff) == 0)
+        assert same.all(), (world, ci)
+        for b in bufs:
+            b.destroy()
