@@ -37,6 +37,7 @@ WORKLOADS = {
     'c1_small': (128, 256, 8, 2, 1, False),
     'c4_decode_zipf': (128, 7168, 256, 8, 128, True),
     'c5_ep32_share': (16384, 7168, 256, 6, 128, True),     # 32 partitions of 8 experts, this GPU = partition 5
+    'c5_ep32_node': (16384, 7168, 256, 6, 128, True),      # all 32 partitions on this GPU, connected
 }
 
 
@@ -169,6 +170,102 @@ def bench_partitioned(args, T, H, E, K, A, R=32, rank=5):
     print(json.dumps(out))
 
 
+def bench_node(args, T, H, E, K, A, R=32, rank=5):
+    """All R partitions of the EP group on this GPU, connected: every partition dispatches T tokens, so each
+    receives its real share (about T*K rows from R sources) and reduces it.  A step runs the four phases for
+    every partition in turn; the phases of one partition are timed with events.  For the record, not the
+    headline line."""
+    import deep_ep
+    dev = torch.device('cuda', 0)
+    x, topk, w = make_inputs(T, H, E, K)
+    xg, tg, wg = x.to(dev), topk.to(dev), w.to(dev)
+    node = deep_ep.LocalNode(R)
+    bufs = [deep_ep.EPBuffer(node.group(r), num_max_tokens_per_rank=T, hidden=H, num_topk=K, use_fp8_dispatch=True,
+                             explicitly_destroy=True) for r in range(R)]
+    kw = dict(num_experts=E, num_max_tokens_per_rank=T, expert_alignment=A, do_expand=True, do_zero_padding=True,
+              fused_fp8_quant=True, async_with_compute_stream=True, defer_epilogue=True)
+    y = None
+    phases = {k: [] for k in ('send', 'recv', 'partial', 'final')}
+
+    def ev():
+        return torch.cuda.Event(enable_timing=True)
+
+    def node_step(timed):
+        nonlocal y
+        marks = [ev() for _ in range(8)]
+        sends = []
+        for r in range(R):
+            if r == rank:
+                marks[0].record()
+            sends.append(bufs[r].dispatch(xg, topk_idx=tg, topk_weights=wg, **kw))
+            if r == rank:
+                marks[1].record()
+        handles, weights = [], []
+        for r in range(R):
+            if r == rank:
+                marks[2].record()
+            (rx, rsf), _, rw, h = sends[r].current_stream_wait()
+            if r == rank:
+                marks[3].record()
+            if y is None or y.size(0) < rx.size(0):
+                y = torch.randn((rx.size(0) + 4096, H), device=dev).to(torch.bfloat16)
+            handles.append(h)
+            weights.append(rw)
+            del rx, rsf
+        partials = []
+        for r in range(R):
+            if r == rank:
+                marks[4].record()
+            partials.append(bufs[r].combine(y[:handles[r].num_expanded_tokens], handles[r], topk_weights=weights[r],
+                                            async_with_compute_stream=True, defer_epilogue=True))
+            if r == rank:
+                marks[5].record()
+        for r in range(R):
+            if r == rank:
+                marks[6].record()
+            partials[r].current_stream_wait()
+            if r == rank:
+                marks[7].record()
+        if timed:
+            torch.cuda.synchronize()
+            for i, k in enumerate(('send', 'recv', 'partial', 'final')):
+                phases[k].append(marks[2 * i].elapsed_time(marks[2 * i + 1]) * 1e3)
+        return handles[rank]
+
+    for _ in range(args.warmup):
+        handle = node_step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        handle = node_step(True)
+    torch.cuda.synchronize()
+    node_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    n_send = int((handle.dst_buffer_slot_idx >= 0).sum())
+    n_recv = int(handle.psum_num_recv_tokens_per_rank[-1])
+    n_valid = int(handle.num_unaligned_recv_tokens_per_expert.sum())
+    tok, ctok = H + 224 + 96, H * 2 + -(-4 * K // 32) * 32
+    nbytes = {'send': T * H * 2 + T * K * 12 + n_send * tok,
+              'recv': n_recv * tok + n_valid * (H + 224 + 4) + 2 * n_recv * (K + 2) * 4 + n_recv * K * 8,
+              'partial': n_valid * H * 2 + n_recv * ctok + n_recv * (K + 2) * 4,
+              'final': n_send * ctok + T * H * 2 + T * K * 12}
+    us = {k: sum(v) / len(v) for k, v in phases.items()}
+    share_ms = node_ms / R
+    out = {'metric': 'dispatch & combine GB/s, one partition of EP32 at its real share (all 32 partitions on one GPU, '
+                     'rows and partials stored straight into peer arenas)',
+           'value': round(sum(nbytes.values()) / share_ms / 1e6, 1), 'unit': 'GB/s', 'n_gpus': 1, 'steps': args.steps,
+           'warmup': args.warmup, 'ms_per_step': round(share_ms, 4), 'higher_is_better': True, 'scaling': 'weak',
+           'vs_baseline': None, 'dtype': 'fp8_e4m3+bf16 payload, fp32 accumulate', 'data': 'synthetic',
+           'config': {'workload': args.workload, 'tokens_per_partition': T, 'hidden': H, 'experts': E, 'topk': K,
+                      'expert_alignment': A, 'partitions': R, 'timed_partition': rank, 'packed_rows_sent': n_send,
+                      'rows_received': n_recv, 'valid_expanded_rows': n_valid, 'node_step_ms': round(node_ms, 3),
+                      'ms_per_step_is': 'node step / partitions (host clock)'},
+           'phases': {k: {'us': round(us[k], 1), 'bytes': nbytes[k], 'gbs': round(nbytes[k] / us[k] / 1e3, 1)}
+                      for k in us}}
+    for b in bufs:
+        b.destroy()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -205,6 +302,9 @@ def main():
         del src, dst
     if args.workload == 'c5_ep32_share':
         bench_partitioned(args, T, H, E, K, A)
+        return
+    if args.workload == 'c5_ep32_node':
+        bench_node(args, T, H, E, K, A)
         return
     x, topk, w = make_inputs(T, H, E, K)
     xg, tg, wg = x.to(dev), topk.to(dev), w.to(dev)

@@ -122,7 +122,7 @@ struct EpScatterArgs {
     int region_by_source;
     int num_ranks;
     int pack_sf_off;              // byte offset of the scales inside a packed row (pack mode)
-    int pad2;
+    int vecs_per_lane;            // verbatim kernel: 16-byte vectors a lane moves per task (1..4)
 };
 
 // recv_sf layouts: rows of scales, or columns of scales whose stride is the row count of recv_sf

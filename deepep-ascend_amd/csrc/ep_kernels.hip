@@ -134,7 +134,9 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(
     short* s_rk = s_key + EP_TOKENS_PER_BLOCK * K;
     int* s_psum = (int*)(s_rk + EP_TOKENS_PER_BLOCK * K);      // [R + waves]  (receive side)
     for (int i = threadIdx.x; i < E + R; i += blockDim.x) smem[i] = 0;
-    layout_load_keys(a, s_key, s_rk, s_psum);
+    const int num_rows = layout_load_keys(a, s_key, s_rk, s_psum);
+    // the scan stops at the last workgroup that has rows: the ones behind it leave nothing
+    if ((int)blockIdx.x > 0 && (int)blockIdx.x * EP_TOKENS_PER_BLOCK >= num_rows) return;
     __syncthreads();
     const int n = EP_TOKENS_PER_BLOCK * K;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -149,15 +151,28 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(
 }
 
 // ------------------------------------------------------------------------------------------------
-// Layout pass B: exclusive prefix over blocks of every histogram column, plus column totals.
-// One workgroup owns 64 columns; its 16 waves split the rows.
+// Layout pass B: exclusive prefix over the workgroups of pass A for every histogram column, plus
+// column totals.  One workgroup owns 16 columns; its 1024 threads are 64 row groups x 16 columns, a
+// thread walks the rows of its group (consecutive threads read consecutive columns of one row).
 // ------------------------------------------------------------------------------------------------
+#define EP_SCAN_COLS 16
+#define EP_SCAN_GROUPS (EP_SCAN_THREADS / EP_SCAN_COLS)
+
 extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpLayoutArgs a) {
-    __shared__ int s_part[EP_SCAN_THREADS / WAVE][WAVE];
-    const int E = a.num_experts, R = a.num_ranks, B = a.num_blocks;
-    const int lane = lane_id(), w = wave_id();
-    const int nw = EP_SCAN_THREADS / WAVE;
-    const int col = blockIdx.x * WAVE + lane;
+    __shared__ int s_part[EP_SCAN_GROUPS][EP_SCAN_COLS + 1];
+    __shared__ int s_rows;
+    const int E = a.num_experts, R = a.num_ranks;
+    int B = a.num_blocks;
+    if (a.recv_mode) {
+        // rows exist only up to the length of the receive stream
+        if (threadIdx.x == 0) s_rows = 0;
+        __syncthreads();
+        if ((int)threadIdx.x < R) atomicAdd(&s_rows, max(0, min(a.inbox[threadIdx.x], a.max_tokens)));
+        __syncthreads();
+        B = min(B, max(1, (s_rows + EP_TOKENS_PER_BLOCK - 1) / EP_TOKENS_PER_BLOCK));
+    }
+    const int c = threadIdx.x % EP_SCAN_COLS, g = threadIdx.x / EP_SCAN_COLS;
+    const int col = blockIdx.x * EP_SCAN_COLS + c;
     const bool live = col < E + R;
     int* base = nullptr;
     int stride = 0;
@@ -165,17 +180,17 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
         if (col < E) { base = a.blk_expert_cnt + col; stride = E; }
         else { base = a.blk_rank_cnt + (col - E); stride = R; }
     }
-    const int rpw = (B + nw - 1) / nw;
-    const int r0 = w * rpw, r1 = min(B, r0 + rpw);
+    const int rpg = (B + EP_SCAN_GROUPS - 1) / EP_SCAN_GROUPS;
+    const int r0 = min(B, g * rpg), r1 = min(B, r0 + rpg);
     int sum = 0;
     if (live)
         for (int r = r0; r < r1; ++r) sum += base[(int64_t)r * stride];
-    s_part[w][lane] = sum;
+    s_part[g][c] = sum;
     __syncthreads();
     int off = 0, total = 0;
-    for (int i = 0; i < nw; ++i) {
-        const int v = s_part[i][lane];
-        if (i < w) off += v;
+    for (int i = 0; i < EP_SCAN_GROUPS; ++i) {
+        const int v = s_part[i][c];
+        if (i < g) off += v;
         total += v;
     }
     if (live) {
@@ -185,7 +200,7 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
             base[(int64_t)r * stride] = run;
             run += v;
         }
-        if (w == 0) {
+        if (g == 0) {
             if (col < E) a.expert_total[col] = total;
             else a.rank_total[col - E] = total;
         }
@@ -228,6 +243,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     // ---- A: stage this block's keys, clear the per-wave counters ----
     for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
     const int num_rows = layout_load_keys(a, s_key, s_rk, s_psum);
+    if (b > 0 && b * EP_TOKENS_PER_BLOCK >= num_rows) return;      // nothing to rank here, nothing to publish
     __syncthreads();
 
     // ---- B: per-wave counts: wave w owns entries [w*epw, (w+1)*epw) of this block's chunk ----
@@ -604,13 +620,24 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
     if (!scatter_row_prologue(a, i, part, c)) return;
     const int K = a.num_topk;
     const int nvec = (int)(a.copy_bytes >> 4);
-    const int v = part * WAVE + lane;
-    if (v < nvec) {
-        const u32x4 d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
-        for (int j = 0; j < K; ++j) {
-            const int s = readlane(c.myslot, j);
-            if (s < 0) continue;
-            __builtin_nontemporal_store(d, (u32x4*)(out_rows_of(a, c, j) + (int64_t)s * a.out_row_bytes) + v);
+    // a task moves vecs_per_lane KiB of the row: 1 where a row fans out to several slots, more where
+    // nearly every row has a single destination and the set-up above would outweigh the copy
+    const int U = a.vecs_per_lane;
+    u32x4 d[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int v = (part * U + u) * WAVE + lane;
+        if (u < U && v < nvec)
+            d[u] = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
+    }
+    for (int j = 0; j < K; ++j) {
+        const int s = readlane(c.myslot, j);
+        if (s < 0) continue;
+        u32x4* row = (u32x4*)(out_rows_of(a, c, j) + (int64_t)s * a.out_row_bytes);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int v = (part * U + u) * WAVE + lane;
+            if (u < U && v < nvec) __builtin_nontemporal_store(d[u], row + v);
         }
     }
     if (part == 0 && a.recv_sf != nullptr) {

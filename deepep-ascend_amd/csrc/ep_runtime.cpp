@@ -559,6 +559,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             sa.region_by_source = b->connected ? 1 : 0;
             sa.num_ranks = num_ranks;
             sa.pack_sf_off = pk.sf_off;
+            sa.vecs_per_lane = 1;
             sa.num_parts = (int)std::max<int64_t>(1, a.fused_fp8_quant ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024));
             sa.num_row_blocks = (int)ceil_div((int64_t)num_tokens * sa.num_parts, EP_ROWS_PER_BLOCK);
             if (sa.num_row_blocks == 0) return;
@@ -627,7 +628,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         if (la.scan_mode != EP_LAYOUT_SINGLE)
             launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, smem_count, a.stream, la);
         if (la.scan_mode == EP_LAYOUT_SCANNED)
-            launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 64), EP_SCAN_THREADS, 0, a.stream, la);
+            launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 16), EP_SCAN_THREADS, 0, a.stream, la);
         launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, a.stream, la);
 
         if (num_ranks > 1) launch_pack();
@@ -725,7 +726,7 @@ int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
         EP_HOST_ASSERT(smem_assign <= 64 * 1024);
         if (la.scan_mode == EP_LAYOUT_SCANNED) {
             launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, layout_count_lds(E, R, K), a.stream, la);
-            launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 64), EP_SCAN_THREADS, 0, a.stream, la);
+            launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 16), EP_SCAN_THREADS, 0, a.stream, la);
         }
         launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, a.stream, la);
         b->last.recv_done = true;
@@ -884,8 +885,11 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
             sa.w_off = pk.w_off;
             quantise_here = false;
         }
-        // a wave task covers 1 KiB of a verbatim row, or 512 channels of a row being quantised
-        sa.num_parts = (int)std::max<int64_t>(1, quantise_here ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024));
+        // a wave task covers 1 KiB of a verbatim row (4 KiB of a packed row, which mostly has one destination
+        // among this partition's few experts), or 512 channels of a row being quantised
+        sa.vecs_per_lane = sa.mode == EP_SCATTER_REGION ? 4 : 1;
+        sa.num_parts = (int)std::max<int64_t>(
+            1, quantise_here ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024 * sa.vecs_per_lane));
         sa.num_row_blocks = (int)ceil_div((int64_t)sa.num_rows_bound * sa.num_parts, EP_ROWS_PER_BLOCK);
         EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0);
         // an expert has at most alignment - 1 padding rows: about one workgroup per 8 of them
