@@ -478,14 +478,16 @@ __device__ __forceinline__ int64_t region_row_of_stream(const int* psum, int R, 
 }
 
 // First byte of the rows that destination j of the task writes, and of their scales.
+template <bool PACK>
 __device__ __forceinline__ char* out_rows_of(const EpScatterArgs& a, const RowCtx& c, int j) {
-    if (a.mode != EP_SCATTER_PACK) return (char*)a.recv_x;
+    if (!PACK) return (char*)a.recv_x;
     const unsigned lo = (unsigned)readlane((int)(unsigned)c.mybase, j);
     const unsigned hi = (unsigned)readlane((int)(unsigned)(c.mybase >> 32), j);
     return (char*)(((uint64_t)hi << 32) | lo);
 }
+template <bool PACK>
 __device__ __forceinline__ char* out_sf_of(const EpScatterArgs& a, char* rows) {
-    return a.mode == EP_SCATTER_PACK ? rows + a.pack_sf_off : (char*)a.recv_sf;
+    return PACK ? rows + a.pack_sf_off : (char*)a.recv_sf;
 }
 
 // A wave task is (row, column part).  Resolves the row's token, its source row and its destination
@@ -499,11 +501,12 @@ __device__ __forceinline__ char* out_sf_of(const EpScatterArgs& a, char* rows) {
 //   EP_SCATTER_REGION  rows of the receive stream (the regions of every source partition in turn), payload,
 //                      scales and weights read from the packed rows; destinations come from the metadata
 //                      rows the receive-side layout wrote (dispatch_copy_epilogue.hpp:459-522)
+template <bool PACK>
 __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int i, int part, RowCtx& c) {
     const int lane = lane_id();
     const int K = a.num_topk;
     int myslot = -1, t;
-    if (a.mode == EP_SCATTER_PACK) {
+    if (PACK) {
         uint64_t mybase = 0;
         t = i;
         int64_t e = -1;
@@ -525,7 +528,7 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
             for (int j = 0; j < K; ++j) {
                 const int g = readlane(myslot, j);
                 if (g < 0) continue;
-                char* row = out_rows_of(a, c, j) + (int64_t)g * a.out_row_bytes;
+                char* row = out_rows_of<PACK>(a, c, j) + (int64_t)g * a.out_row_bytes;
                 if (lane < K) {
                     if (a.with_metadata) ((int64_t*)(row + a.idx_off))[lane] = e;
                     ((float*)(row + a.w_off))[lane] = w;
@@ -606,7 +609,8 @@ __device__ __forceinline__ void zero_padding_rows(const EpScatterArgs& a) {
 // Verbatim rows: BF16 payload, or FP8 payload with its 2-byte scale packs.  A task moves 1 KiB of
 // the row (16 bytes per lane) to every slot; many short tasks keep far more loads in flight than
 // one wave walking a whole row.
-extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpScatterArgs a) {
+template <bool PACK>
+__device__ __forceinline__ void scatter_copy_body(const EpScatterArgs& a) {
     if ((int)blockIdx.x >= a.num_row_blocks) {
         zero_padding_rows(a);
         return;
@@ -617,7 +621,7 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
     const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
     if (i >= n) return;
     RowCtx c;
-    if (!scatter_row_prologue(a, i, part, c)) return;
+    if (!scatter_row_prologue<PACK>(a, i, part, c)) return;
     const int K = a.num_topk;
     const int nvec = (int)(a.copy_bytes >> 4);
     // a task moves vecs_per_lane KiB of the row: 1 where a row fans out to several slots, more where
@@ -633,7 +637,7 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
     for (int j = 0; j < K; ++j) {
         const int s = readlane(c.myslot, j);
         if (s < 0) continue;
-        u32x4* row = (u32x4*)(out_rows_of(a, c, j) + (int64_t)s * a.out_row_bytes);
+        u32x4* row = (u32x4*)(out_rows_of<PACK>(a, c, j) + (int64_t)s * a.out_row_bytes);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int v = (part * U + u) * WAVE + lane;
@@ -648,7 +652,7 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
             for (int j = 0; j < K; ++j) {
                 const int s = readlane(c.myslot, j);
                 if (s < 0) continue;
-                ((unsigned short*)(out_sf_of(a, out_rows_of(a, c, j)) + (int64_t)s * a.out_sf_row_bytes))[p] = val;
+                ((unsigned short*)(out_sf_of<PACK>(a, out_rows_of<PACK>(a, c, j)) + (int64_t)s * a.out_sf_row_bytes))[p] = val;
             }
         }
     }
@@ -657,7 +661,14 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpS
 // Fused BF16 -> e4m3fn quantisation (deep_ep/utils/math.py:30-38) + scatter.  A task owns 512
 // channels of a row: a lane holds 8 of them, a 128-channel group is one DPP row of 16 lanes, so the
 // task produces 512 payload bytes and 4 fp32 scales per slot.
-template <bool HW>
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy(EpScatterArgs a) {
+    scatter_copy_body<false>(a);
+}
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy_pack(EpScatterArgs a) {
+    scatter_copy_body<true>(a);
+}
+
+template <bool HW, bool PACK>
 __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     if ((int)blockIdx.x >= a.num_row_blocks) {
         zero_padding_rows(a);
@@ -669,7 +680,7 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
     if (i >= n) return;
     RowCtx c;
-    if (!scatter_row_prologue(a, i, part, c)) return;
+    if (!scatter_row_prologue<PACK>(a, i, part, c)) return;
     const int K = a.num_topk;
     const int nvec = a.hidden >> 3;                      // 16-byte vectors of 8 BF16
     const int v = part * WAVE + lane;
@@ -691,17 +702,23 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     for (int j = 0; j < K; ++j) {
         const int s = readlane(c.myslot, j);
         if (s < 0) continue;
-        char* rows = out_rows_of(a, c, j);
+        char* rows = out_rows_of<PACK>(a, c, j);
         __builtin_nontemporal_store(q8, (u32x2*)(rows + (int64_t)s * a.out_row_bytes) + v);
-        if (writes_scale) ((float*)(out_sf_of(a, rows) + (int64_t)s * a.out_sf_row_bytes))[v >> 4] = scale;
+        if (writes_scale) ((float*)(out_sf_of<PACK>(a, rows) + (int64_t)s * a.out_sf_row_bytes))[v >> 4] = scale;
     }
 }
 
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant(EpScatterArgs a) {
-    scatter_quant_body<true>(a);
+    scatter_quant_body<true, false>(a);
 }
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_sw(EpScatterArgs a) {
-    scatter_quant_body<false>(a);
+    scatter_quant_body<false, false>(a);
+}
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_pack(EpScatterArgs a) {
+    scatter_quant_body<true, true>(a);
+}
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_sw_pack(EpScatterArgs a) {
+    scatter_quant_body<false, true>(a);
 }
 
 // Column-major scales (use_tma_aligned_col_major_sf): the copy kernels write scale rows, this

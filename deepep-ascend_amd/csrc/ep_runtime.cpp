@@ -110,6 +110,7 @@ struct Kernels {
     hipModule_t module = nullptr;
     hipFunction_t layout_count, layout_scan, layout_assign;
     hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw, sf_transpose;
+    hipFunction_t scatter_copy_pack, scatter_quant_pack, scatter_quant_sw_pack;
     hipFunction_t combine[3][5];     // [mode][generic, k2, k4, k6, k8]
     hipFunction_t fp8_selftest;
     int device = -1;
@@ -147,6 +148,9 @@ void load_kernels(const char* dir) {
     get(g_k.scatter_copy, "ep_scatter_copy");
     get(g_k.scatter_quant, "ep_scatter_quant");
     get(g_k.scatter_quant_sw, "ep_scatter_quant_sw");
+    get(g_k.scatter_copy_pack, "ep_scatter_copy_pack");
+    get(g_k.scatter_quant_pack, "ep_scatter_quant_pack");
+    get(g_k.scatter_quant_sw_pack, "ep_scatter_quant_sw_pack");
     get(g_k.sf_transpose, "ep_sf_transpose");
     const char* modes[3] = {"", "_partial", "_final"};
     const char* ks[5] = {"_generic", "_k2", "_k4", "_k6", "_k8"};
@@ -563,7 +567,8 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             sa.num_parts = (int)std::max<int64_t>(1, a.fused_fp8_quant ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024));
             sa.num_row_blocks = (int)ceil_div((int64_t)num_tokens * sa.num_parts, EP_ROWS_PER_BLOCK);
             if (sa.num_row_blocks == 0) return;
-            hipFunction_t fn = a.fused_fp8_quant ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
+            hipFunction_t fn = a.fused_fp8_quant ? (g_fp8_hw ? g_k.scatter_quant_pack : g_k.scatter_quant_sw_pack)
+                                                 : g_k.scatter_copy_pack;
             launch(fn, (unsigned)sa.num_row_blocks, EP_ROW_THREADS, 0, a.stream, sa);
         };
 
