@@ -3,9 +3,14 @@
 //
 // Kernels (all HBM-bound, no MFMA):
 //   ep_layout_count / ep_layout_scan / ep_layout_assign   stable counting sort of the (token, slot)
-//       entries by destination partition and by local expert -> every handle tensor
+//       entries by destination partition and by local expert -> every handle tensor; with several
+//       partitions once on the send side (slots in the destinations' regions) and once on the receive
+//       side (slots of the rows that arrived)
 //   ep_scatter_copy / ep_scatter_quant                     receive-stream row -> its expanded slots
+//   ep_scatter_copy_pack / ep_scatter_quant_pack           token -> one packed row per destination partition
+//   ep_sf_transpose                                        scale rows -> scale columns
 //   ep_combine_k<K> / ep_combine_generic                   K-way gather + fp32 reduce back to token order
+//   ep_combine_partial_* / ep_combine_final_*              the same reduce in its owner-side and token-side halves
 //   ep_fp8_selftest                                        hardware vs integer e4m3fn conversion
 #include <hip/hip_runtime.h>
 #include <stdint.h>
