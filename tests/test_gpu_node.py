@@ -128,6 +128,23 @@ def test_node_dispatch_combine(R, max_tokens, H, E, K, A, masked, mode, do_cpu_s
         assert np.array_equal(rw.cpu().numpy().view(np.uint32)[:ne], want[r]['w'].view(np.uint32))
         handles.append(handle)
 
+    # cached replay through the node: new payload and weights, the layout of the handles
+    if mode == 'bf16' and do_cpu_sync:
+        xs2 = [make_tokens(T, H, seed=30 * R + r) for r, T in enumerate(Ts)]
+        ws2 = [torch.randn(w.shape, generator=torch.Generator().manual_seed(r)).masked_fill(topks[r] < 0, 0)
+               for r, w in enumerate(ws)]
+        rows2 = [bf16_bits(x).view(np.uint8).reshape(x.size(0), -1) for x in xs2]
+        _, want2 = oracle_dispatch(rows2, sfs, [t.numpy() for t in topks], [w.numpy() for w in ws2], E, R, A, max_tokens)
+        evs = [bufs[r].dispatch(xs2[r].to(DEV), topk_weights=ws2[r].to(DEV), handle=handles[r], do_expand=True,
+                                do_zero_padding=True, async_with_compute_stream=True, defer_epilogue=True)
+               for r in range(R)]
+        outs2 = [ev.current_stream_wait() for ev in evs]
+        torch.cuda.synchronize()
+        for r, (rx2, _, rw2, h2) in enumerate(outs2):
+            assert h2 is handles[r]
+            assert np.array_equal(rx2.view(torch.uint8).cpu().numpy().reshape(rx2.size(0), -1), want2[r]['x'])
+            assert np.array_equal(rw2.cpu().numpy().view(np.uint32), want2[r]['w'].view(np.uint32))
+
     # combine: every owner reduces what it received and sends the partial home
     g = torch.Generator().manual_seed(R)
     ys = [torch.randn((outs[r][0][0].size(0) if isinstance(outs[r][0], tuple) else outs[r][0].size(0), H),

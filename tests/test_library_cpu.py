@@ -146,6 +146,8 @@ int main(void) {
     printf("%zu %zu %zu %zu\\n", offsetof(ep_dispatch_args_t, stream), offsetof(ep_dispatch_args_t, fused_fp8_quant),
            offsetof(ep_dispatch_epilogue_args_t, stream), offsetof(ep_dispatch_epilogue_args_t, recv_sf_layout));
     printf("%zu %zu\\n", offsetof(ep_combine_args_t, stream), offsetof(ep_combine_args_t, apply_weights));
+    printf("%zu %zu %zu\\n", sizeof(ep_dispatch_recv_args_t), offsetof(ep_dispatch_recv_args_t, stream),
+           offsetof(ep_dispatch_recv_args_t, hidden_bytes));
     return 0;
 }
 ''')
@@ -157,5 +159,7 @@ int main(void) {
            ctypes.sizeof(C._CombineArgs),
            C._DispatchArgs.stream.offset, C._DispatchArgs.fused_fp8_quant.offset,
            C._DispatchEpilogueArgs.stream.offset, C._DispatchEpilogueArgs.recv_sf_layout.offset,
-           C._CombineArgs.stream.offset, C._CombineArgs.apply_weights.offset]
+           C._CombineArgs.stream.offset, C._CombineArgs.apply_weights.offset,
+           ctypes.sizeof(C._DispatchRecvArgs), C._DispatchRecvArgs.stream.offset,
+           C._DispatchRecvArgs.hidden_bytes.offset]
     assert got == [int(v) for v in out]
