@@ -1,7 +1,8 @@
-"""Builds the two native artefacts of the package for gfx950, in-tree:
+"""Builds the native artefacts of the package for gfx950, in-tree:
 
   deep_ep/lib/ep_kernels.hsaco     device code object   (hipcc --genco)
   deep_ep/lib/libdeep_ep_hip.so    host runtime, C ABI  (hipcc -shared)
+  deep_ep/lib/abi_client           a plain-C caller of the C ABI, used by the tests  (gcc)
 
 hipcc cross-compiles, so this runs on a machine without a GPU.  `python deepep-ascend_amd/deep_ep/_build.py`.
 """
@@ -21,6 +22,8 @@ DEVICE_FLAGS = [
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
 ]
 HOST_FLAGS = ['-shared', '-fPIC', '-O2', '-std=c++17', '-Wall']
+ROCM = os.environ.get('ROCM_PATH', '/opt/rocm')
+C_CLIENT_FLAGS = ['-std=c11', '-O1', '-Wall', '-D__HIP_PLATFORM_AMD__', f'-I{ROCM}/include']
 
 
 def run(cmd):
@@ -32,6 +35,8 @@ def build(verbose: bool = True) -> None:
     os.makedirs(LIB, exist_ok=True)
     run([HIPCC, *DEVICE_FLAGS, '-o', os.path.join(LIB, 'ep_kernels.hsaco'), os.path.join(CSRC, 'ep_kernels.hip')])
     run([HIPCC, *HOST_FLAGS, '-o', os.path.join(LIB, 'libdeep_ep_hip.so'), os.path.join(CSRC, 'ep_runtime.cpp')])
+    run(['gcc', *C_CLIENT_FLAGS, '-o', os.path.join(LIB, 'abi_client'), os.path.join(CSRC, 'abi_client.c'),
+         f'-L{LIB}', '-ldeep_ep_hip', f'-L{ROCM}/lib', '-lamdhip64', '-Wl,-rpath,$ORIGIN', f'-Wl,-rpath,{ROCM}/lib'])
 
 
 if __name__ == '__main__':

@@ -233,3 +233,16 @@ def test_single_and_multi_block_layouts_agree_with_oracle(T, E, K, R, rank):
         assert np.array_equal(getattr(handle, name).cpu().numpy(), lay[name]), name
     assert handle.num_recv_tokens_per_expert_list == lay['num_recv_tokens_per_expert_list']
     buf.destroy()
+
+
+def test_plain_c_caller_of_the_abi():
+    """deep_ep/lib/abi_client (csrc/abi_client.c, built with gcc): the C ABI used without torch or C++,
+    with hipMalloc'd tensors and its own stream; it checks the layout and an exact round trip itself."""
+    import os
+    import subprocess
+    import deep_ep
+    exe = os.path.join(os.path.dirname(deep_ep.__file__), 'lib', 'abi_client')
+    assert os.path.exists(exe), 'run deep_ep/_build.py'
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr
+    assert res.stdout.startswith('abi_client: ok')
