@@ -256,3 +256,42 @@ def test_node_reproduces_the_reference_combine_vectors(world):
         assert same.all(), (world, ci)
         for b in bufs:
             b.destroy()
+
+
+def test_node_with_an_empty_partition_and_disconnect():
+    """A partition without tokens still takes part (it receives and reduces for the others); destroying a
+    partition leaves the rest usable on their own."""
+    R, max_tokens, H, E, K, A = 2, 40, 128, 4, 2, 4
+    bufs = make_node(R, max_tokens, H, K, False)
+    Ts = [33, 0]
+    xs = [make_tokens(T, H, seed=r) if T else torch.empty((0, H), dtype=torch.bfloat16) for r, T in enumerate(Ts)]
+    routing = [make_routing(T, E, K, seed=r) if T else (torch.empty((0, K), dtype=torch.int64),
+                                                         torch.empty((0, K), dtype=torch.float32))
+               for r, T in enumerate(Ts)]
+    topks, ws = [t for t, _ in routing], [w for _, w in routing]
+    rows = [bf16_bits(x).view(np.uint8).reshape(x.size(0), H * 2) for x in xs]
+    _, want = oracle_dispatch(rows, [None] * R, [t.numpy() for t in topks], [w.numpy() for w in ws], E, R, A, max_tokens)
+    outs = dispatch_all(bufs, [x.to(DEV) for x in xs], [t.to(DEV) for t in topks], [w.to(DEV) for w in ws],
+                        num_experts=E, num_max_tokens_per_rank=max_tokens, expert_alignment=A, do_expand=True,
+                        do_zero_padding=True)
+    torch.cuda.synchronize()
+    for r, (rx, _, rw, handle) in enumerate(outs):
+        assert np.array_equal(handle.recv_src_metadata.cpu().numpy(), want[r]['lay']['recv_src_metadata'])
+        assert np.array_equal(rx.view(torch.uint8).cpu().numpy().reshape(rx.size(0), H * 2), want[r]['x'])
+    ys = [o[0] for o in outs]                                   # identity experts
+    res = combine_all(bufs, ys, [o[3] for o in outs], [o[2] for o in outs], [None] * R)
+    torch.cuda.synchronize()
+    # every token selected K distinct experts: the sum of K copies
+    expect = (xs[0].float() * K).to(torch.bfloat16)
+    assert torch.equal(res[0][0].cpu().view(torch.int16), expect.view(torch.int16))
+    assert torch.equal(res[0][1].cpu(), ws[0]) and res[1][0].size(0) == 0
+
+    bufs[1].destroy()
+    x = xs[0].to(DEV)
+    rx, _, rw, handle, _ = bufs[0].dispatch(x, topk_idx=topks[0].to(DEV), topk_weights=ws[0].to(DEV), num_experts=E,
+                                            num_max_tokens_per_rank=max_tokens, expert_alignment=A, do_expand=True,
+                                            do_zero_padding=True)
+    torch.cuda.synchronize()
+    lay = O.rank_share_layout(topks[0].numpy(), E, R, 0, A, max_tokens)
+    assert np.array_equal(handle.recv_src_metadata.cpu().numpy(), lay['recv_src_metadata'])
+    bufs[0].destroy()
