@@ -238,3 +238,123 @@ def test_dispatch_combine_flow(do_cpu_sync, defer_epilogue, masked):
             else:
                 assert ccw is None
     buf.destroy()
+
+
+@pytest.mark.parametrize('R', [2, 4])
+def test_node_flow(R):
+    """The same properties with every rank of the group present (a node of R partitions on this GPU), ragged
+    token counts `max(1, N - rank)` as tests/ep/test_ep.py:53: what each partition receives is checked against
+    the tokens the *other* partitions hold, and the combine against sums over all partitions' experts."""
+    de = _deep_ep()
+    max_tokens, H, E, K = 120, 256, 16, 4
+    El = E // R
+    node = de.LocalNode(R)
+    bufs = [de.EPBuffer(node.group(r), num_max_tokens_per_rank=max_tokens, hidden=H, num_topk=K,
+                        use_fp8_dispatch=True, explicitly_destroy=True) for r in range(R)]
+    Ts = [max(1, max_tokens - r) for r in range(R)]
+    routing = [make_routing(T, E, K, seed=40 + r, masked=0.2) for r, T in enumerate(Ts)]
+    topk = [t.to(DEV) for t, _ in routing]
+    wts = [w.to(DEV) for _, w in routing]
+
+    for alignment, num_bias, fp8, col_major in dispatch_modes():
+        if num_bias == 1:
+            continue
+        g = torch.Generator(device=DEV).manual_seed(alignment + num_bias)
+        xs = [torch.randn((T, H), device=DEV, generator=g).to(torch.bfloat16) for T in Ts]
+        if fp8:
+            pairs = [de.utils.math.per_token_cast_to_fp8(x) for x in xs]
+            x_args = [(q, s.view(torch.int16)) for q, s in pairs]
+            ref_rows = [q.view(torch.uint8) for q, _ in pairs]
+            ref_sfs = [s.view(torch.int16) for _, s in pairs]
+        else:
+            x_args, ref_rows, ref_sfs = xs, xs, [None] * R
+        biases = [tuple(torch.randn((T, H), device=DEV, generator=g).to(torch.bfloat16) for _ in range(2))
+                  if num_bias else None for T in Ts]
+
+        events = [bufs[r].dispatch(x_args[r], topk_idx=topk[r], topk_weights=wts[r], num_experts=E,
+                                   num_max_tokens_per_rank=max_tokens, expert_alignment=alignment, do_expand=True,
+                                   do_zero_padding=True, use_tma_aligned_col_major_sf=col_major,
+                                   async_with_compute_stream=True, defer_epilogue=True) for r in range(R)]
+        outs = [ev.current_stream_wait(release_handle=True) for ev in events]
+        torch.cuda.synchronize()
+
+        y3 = [torch.randn((T, K, H), device=DEV, generator=g).to(torch.bfloat16) for T in Ts]   # expert outputs
+        ys = []
+        for d, (recv, _, rw, handle) in enumerate(outs):
+            recv_data, recv_sf = recv if fp8 else (recv, None)
+            check_x = recv_data.view(torch.uint8) if fp8 else recv_data
+            n_exp = recv_data.size(0)
+            meta = handle.recv_src_metadata
+            src, slots, master = meta[:, -2].long(), meta[:, :-2], meta[:, -1]
+            src_rank, src_tok = src // max_tokens, src % max_tokens
+            # per source: its tokens with a selection on partition d, each once, sources in rank order
+            psum = [0] + handle.psum_num_recv_tokens_per_rank.tolist()
+            for s in range(R):
+                local = (topk[s] >= d * El) & (topk[s] < (d + 1) * El)
+                part = slice(psum[s], psum[s + 1])
+                assert torch.equal(src_rank[part], torch.full_like(src_rank[part], s))
+                assert torch.equal(torch.sort(src_tok[part]).values, local.any(dim=1).nonzero().flatten())
+            all_topk = torch.cat([torch.nn.functional.pad(t, (0, 0, 0, max_tokens - t.size(0)), value=-1) for t in topk])
+            sel = all_topk[src]                                         # global expert ids of every received row
+            local = (sel >= d * El) & (sel < (d + 1) * El)
+            assert torch.equal(slots >= 0, local)
+            flat = slots[local].long()
+            assert flat.numel() == handle.num_unaligned_recv_tokens_per_expert.sum().item()
+            assert torch.unique(flat).numel() == flat.numel() and (flat.numel() == 0 or flat.max().item() < n_exp)
+            all_rows = torch.cat([torch.nn.functional.pad(r_, (0, 0, 0, max_tokens - r_.size(0))) for r_ in ref_rows])
+            assert torch.equal(check_x[flat], all_rows[src].unsqueeze(1).expand(-1, K, -1)[local])
+            if fp8:
+                assert recv_sf.stride() == ((1, n_exp) if col_major else (recv_sf.size(1), 1))
+                all_sf = torch.cat([torch.nn.functional.pad(s_, (0, 0, 0, max_tokens - s_.size(0))) for s_ in ref_sfs])
+                assert torch.equal(recv_sf[flat], all_sf[src].unsqueeze(1).expand(-1, K, -1)[local])
+            all_w = torch.cat([torch.nn.functional.pad(w_, (0, 0, 0, max_tokens - w_.size(0))) for w_ in wts])
+            assert torch.equal(rw[flat], all_w[src][local])
+            pos = torch.arange(K, device=DEV, dtype=meta.dtype).view(1, K)
+            assert torch.equal(master, torch.where(local, pos, torch.full_like(slots, -1)).max(dim=1).values)
+            pe = [0] + handle.psum_num_recv_tokens_per_expert.tolist()
+            for e in range(El):
+                start, end = _align(pe[e], alignment), pe[e + 1]
+                assert end - start == sum(int((t == d * El + e).sum()) for t in topk)
+                mine = torch.sort(slots[sel == d * El + e]).values
+                assert torch.equal(mine, torch.arange(start, end, device=DEV, dtype=mine.dtype))
+                assert torch.count_nonzero(recv_data[end:_align(end, alignment)].view(torch.uint8)).item() == 0
+            # expert output of (source token, j) at its slot, garbage elsewhere
+            y = torch.randn((n_exp, H), device=DEV, generator=g).to(torch.bfloat16) * 100
+            all_y3 = torch.cat([torch.nn.functional.pad(v, (0, 0, 0, 0, 0, max_tokens - v.size(0))) for v in y3])
+            if flat.numel():
+                y[flat] = all_y3[src][local]
+            ys.append(y)
+
+        cevs = [bufs[r].combine(ys[r], outs[r][3], topk_weights=outs[r][2], bias=biases[r],
+                                async_with_compute_stream=True, defer_epilogue=True) for r in range(R)]
+        res = [ev.current_stream_wait(release_handle=True) for ev in cevs]
+        torch.cuda.synchronize()
+        for s in range(R):
+            # one BF16 partial per destination partition (fp32 sum in ascending position), then biases and
+            # partials in ascending position of each partition's last selection (refs.py:175-250)
+            T = Ts[s]
+            rank_of = torch.where(topk[s] >= 0, topk[s] // El, torch.full_like(topk[s], -1))
+            partial = torch.zeros((T, K, H), dtype=torch.float32, device=DEV)        # indexed by master position
+            is_master = torch.zeros((T, K), dtype=torch.bool, device=DEV)
+            for j in range(K):
+                later_same = torch.zeros(T, dtype=torch.bool, device=DEV)
+                for jj in range(j + 1, K):
+                    later_same |= (rank_of[:, jj] == rank_of[:, j])
+                is_master[:, j] = (rank_of[:, j] >= 0) & ~later_same
+                acc = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+                for jj in range(j + 1):
+                    same = (rank_of[:, jj] == rank_of[:, j]) & (rank_of[:, j] >= 0)
+                    acc = acc + torch.where(same.unsqueeze(1), y3[s][:, jj].float(), torch.zeros_like(acc))
+                partial[:, j] = acc.to(torch.bfloat16).float()
+            total = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+            if biases[s] is not None:
+                total = biases[s][0].float() + biases[s][1].float()
+            for j in range(K):
+                total = total + torch.where(is_master[:, j:j + 1], partial[:, j], torch.zeros_like(total))
+            want = total.to(torch.bfloat16)
+            cx, cw = res[s]
+            same = (cx.view(torch.int16) == want.view(torch.int16)) | ((cx == 0) & (want == 0))   # sign of zero
+            assert bool(same.all()), (alignment, num_bias, fp8, col_major, s)
+            assert torch.equal(cw, wts[s])
+    for b in bufs:
+        b.destroy()
