@@ -1,25 +1,33 @@
-from abc import ABC, abstractmethod
+"""What every communication buffer shares: it owns one native runtime object, and that object is
+released either by an explicit `destroy()` or together with its owner (reference:
+deep_ep/buffers/base.py, csrc/buffers/base.hpp)."""
+import abc
 
 
-class BufferBase(ABC):
-    """Lifecycle shared by the communication buffers: a native runtime object that is either
-    destroyed explicitly or with its owner."""
+class BufferBase(abc.ABC):
+    runtime = None
 
     def __init__(self, explicitly_destroy: bool = False):
-        self.explicitly_destroy = explicitly_destroy
-        self.runtime = None
+        self.explicitly_destroy = bool(explicitly_destroy)
+
+    def _runtime_or_fail(self):
+        if self.runtime is None:
+            raise AssertionError('the buffer has been destroyed')
+        return self.runtime
 
     @property
     def main_context(self):
-        return None if self.runtime is None else self.runtime.main_context
+        runtime = self.runtime
+        return runtime.main_context if runtime is not None else None
 
     def print_memory_usage(self) -> None:
-        assert self.runtime is not None
-        self.runtime.print_memory_usage()
+        self._runtime_or_fail().print_memory_usage()
 
-    @abstractmethod
+    @abc.abstractmethod
     def destroy(self) -> None:
-        assert self.explicitly_destroy
+        """Only buffers built with `explicitly_destroy=True` may be destroyed by hand."""
+        if not self.explicitly_destroy:
+            raise AssertionError('explicitly_destroy=True is required to call destroy()')
         runtime, self.runtime = self.runtime, None
         if runtime is not None:
             runtime.destroy()

@@ -41,26 +41,21 @@ class EPHandle:
             output (upper bounds when the dispatch did not sync with the host).
     """
 
+    _CALL_FIELDS = ('do_expand', 'num_experts', 'expert_alignment', 'num_max_tokens_per_rank', 'num_sms')
+    _LAYOUT_FIELDS = ('num_recv_tokens', 'num_expanded_tokens', 'num_recv_tokens_per_expert_list',
+                      'psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
+                      'num_unaligned_recv_tokens_per_expert', 'recv_src_metadata', 'dst_buffer_slot_idx',
+                      'dst_gsge_idx')
+
     def __init__(self, do_expand: bool, num_experts: int, expert_alignment: int, num_max_tokens_per_rank: int,
                  num_sms: int, topk_idx: torch.Tensor, num_recv_tokens: int, num_expanded_tokens: int,
                  num_recv_tokens_per_expert_list: list, psum_num_recv_tokens_per_rank: torch.Tensor,
                  psum_num_recv_tokens_per_expert: torch.Tensor, num_unaligned_recv_tokens_per_expert: torch.Tensor,
                  recv_src_metadata: torch.Tensor, dst_buffer_slot_idx: torch.Tensor, dst_gsge_idx: torch.Tensor):
         assert topk_idx is not None
-        self.do_expand = do_expand
-        self.num_experts = num_experts
-        self.expert_alignment = expert_alignment
-        self.num_max_tokens_per_rank = num_max_tokens_per_rank
-        self.num_sms = num_sms
-        self.num_recv_tokens = num_recv_tokens
-        self.num_expanded_tokens = num_expanded_tokens
-        self.num_recv_tokens_per_expert_list = num_recv_tokens_per_expert_list
-        self.psum_num_recv_tokens_per_rank = psum_num_recv_tokens_per_rank
-        self.psum_num_recv_tokens_per_expert = psum_num_recv_tokens_per_expert
-        self.num_unaligned_recv_tokens_per_expert = num_unaligned_recv_tokens_per_expert
-        self.recv_src_metadata = recv_src_metadata
-        self.dst_buffer_slot_idx = dst_buffer_slot_idx
-        self.dst_gsge_idx = dst_gsge_idx
+        given = locals()
+        for name in self._CALL_FIELDS + self._LAYOUT_FIELDS:
+            setattr(self, name, given[name])
         self.cached_recv_src_metadata_before_sort = None
         self._topk_idx = topk_idx
         # inference tensors carry no version counter
@@ -95,76 +90,70 @@ class EPBuffer(BufferBase):
     get_physical_domain_size = comm.get_physical_domain_size
     get_logical_domain_size = comm.get_logical_domain_size
 
-    def __init__(self,
-                 group,
-                 num_bytes: Optional[int] = None,
-                 num_max_tokens_per_rank: int = 0,
-                 hidden: int = 0,
-                 num_topk: int = 0,
-                 use_fp8_dispatch: bool = False,
-                 lb_allocation_plan_or_num_bytes: Union[BufferAllocator, int] = 0,
-                 deterministic: bool = False,
-                 allow_hybrid_mode: bool = True,
-                 allow_multiple_reduction: bool = True,
-                 prefer_overlap_with_compute: bool = True,
-                 sl_idx: Optional[int] = None,
-                 num_allocated_qps: int = 0,
-                 num_cpu_timeout_secs: int = 300, num_gpu_timeout_secs: int = 100,
-                 explicitly_destroy: bool = False,
+    def __init__(self, group, num_bytes: Optional[int] = None, num_max_tokens_per_rank: int = 0, hidden: int = 0,
+                 num_topk: int = 0, use_fp8_dispatch: bool = False,
+                 lb_allocation_plan_or_num_bytes: Union[BufferAllocator, int] = 0, deterministic: bool = False,
+                 allow_hybrid_mode: bool = True, allow_multiple_reduction: bool = True,
+                 prefer_overlap_with_compute: bool = True, sl_idx: Optional[int] = None, num_allocated_qps: int = 0,
+                 num_cpu_timeout_secs: int = 300, num_gpu_timeout_secs: int = 100, explicitly_destroy: bool = False,
                  *, use_huge1g_page: bool = True):
         """`group` needs `rank()` and `size()`.  `num_bytes` (without workspace) must be a multiple
         of `get_num_allocation_alignment()`; when None it comes from `get_buffer_size_hint`.
         Load-balancing storage can be reserved; the load-balancing kernels, RDMA service levels
         and explicit QP counts do not exist here."""
-        plan = lb_allocation_plan_or_num_bytes if isinstance(lb_allocation_plan_or_num_bytes, BufferAllocator) else None
-        num_lb_bytes = plan.num_bytes if plan is not None else lb_allocation_plan_or_num_bytes
-        if plan is not None:
-            assert not plan.materialized
-        assert isinstance(num_lb_bytes, int) and num_lb_bytes >= 0
-        assert num_lb_bytes % _C.get_num_allocation_alignment() == 0
         if sl_idx is not None or num_allocated_qps != 0:
             raise NotImplementedError('RDMA service levels and QP configuration are not implemented')
-        assert allow_multiple_reduction, 'allow_multiple_reduction=True is required'
-        assert num_cpu_timeout_secs > 0 and num_gpu_timeout_secs > 0
+        if not allow_multiple_reduction:
+            raise AssertionError('allow_multiple_reduction=True is required')
+        if min(num_cpu_timeout_secs, num_gpu_timeout_secs) <= 0:
+            raise AssertionError('time-outs are positive numbers of seconds')
+        granule = _C.get_num_allocation_alignment()
 
-        self.group = group
-        self.rank_idx, self.num_ranks = group.rank(), group.size()
-        self.allow_hybrid_mode = allow_hybrid_mode
-        self.allow_multiple_reduction = allow_multiple_reduction
-        self.prefer_overlap_with_compute = prefer_overlap_with_compute
-        self.deterministic = deterministic
-        self.num_max_tokens_per_rank = num_max_tokens_per_rank
-        self.num_allocated_qps = 0
-        self.num_lb_bytes = num_lb_bytes
+        # load-balancing storage: a byte count, or a plan whose tensors get their memory below
+        lb_plan = lb_allocation_plan_or_num_bytes
+        if isinstance(lb_plan, BufferAllocator):
+            assert not lb_plan.materialized, 'the allocation plan already has storage'
+            num_lb_bytes = lb_plan.num_bytes
+        else:
+            lb_plan, num_lb_bytes = None, lb_allocation_plan_or_num_bytes
+        if not isinstance(num_lb_bytes, int) or num_lb_bytes < 0 or num_lb_bytes % granule:
+            raise AssertionError(f'load-balancing storage must be a non-negative multiple of {granule} bytes')
+
         if num_bytes is None:
-            num_bytes = self.get_buffer_size_hint(group, num_max_tokens_per_rank, hidden, num_topk,
-                                                  use_fp8_dispatch, allow_hybrid_mode, allow_multiple_reduction)
-        assert num_bytes >= 0 and num_bytes % _C.get_num_allocation_alignment() == 0
-        self.num_bytes = num_bytes
-        if os.environ.get('EP_BUFFER_DEBUG', 0):
-            print(f'Initializing EP buffer with {num_bytes} bytes at rank EP {self.rank_idx}/{self.num_ranks}')
+            num_bytes = self.get_buffer_size_hint(group, num_max_tokens_per_rank, hidden, num_topk, use_fp8_dispatch,
+                                                  allow_hybrid_mode, allow_multiple_reduction)
+        if num_bytes < 0 or num_bytes % granule:
+            raise AssertionError(f'num_bytes must be a non-negative multiple of {granule}')
 
-        self.hccl_comm_handle = comm.get_hccl_comm_handle(group)
         super().__init__(explicitly_destroy)
-        self.runtime = _C.EPBuffer(self.rank_idx, self.num_ranks, self.hccl_comm_handle.get(), num_bytes,
-                                   num_lb_bytes, use_huge1g_page, num_cpu_timeout_secs, num_gpu_timeout_secs,
-                                   explicitly_destroy)
+        rank_idx, num_ranks = group.rank(), group.size()
+        vars(self).update(
+            group=group, rank_idx=rank_idx, num_ranks=num_ranks, num_bytes=num_bytes, num_lb_bytes=num_lb_bytes,
+            num_max_tokens_per_rank=num_max_tokens_per_rank, deterministic=deterministic, num_allocated_qps=0,
+            allow_hybrid_mode=allow_hybrid_mode, allow_multiple_reduction=allow_multiple_reduction,
+            prefer_overlap_with_compute=prefer_overlap_with_compute,
+            hccl_comm_handle=comm.get_hccl_comm_handle(group))
+        if os.environ.get('EP_BUFFER_DEBUG'):
+            print(f'EP buffer of partition {rank_idx}/{num_ranks}: {num_bytes} bytes + {num_lb_bytes} bytes of storage')
+
+        self.runtime = _C.EPBuffer(rank_idx, num_ranks, self.hccl_comm_handle.get(), num_bytes, num_lb_bytes,
+                                   use_huge1g_page, num_cpu_timeout_secs, num_gpu_timeout_secs, explicitly_destroy)
         self.context = self.runtime.context
         node = getattr(group, 'node', None)
         if node is not None:
-            node.register(self.rank_idx, self.runtime)      # the last partition of a node connects them all
-        if plan is not None:
-            plan.materialize(self.runtime.lb_storage)
+            node.register(rank_idx, self.runtime)           # the last partition of a node connects them all
+        if lb_plan is not None:
+            lb_plan.materialize(self.runtime.lb_storage)
+
+        # everything is directly addressable here: one "scale-out" domain holding all partitions
         self.num_scaleout_ranks, self.num_scaleup_ranks = self.get_logical_domain_size()
-        self.scaleout_rank_idx = self.rank_idx // self.num_scaleup_ranks
-        self.scaleup_rank_idx = self.rank_idx % self.num_scaleup_ranks
+        self.scaleout_rank_idx, self.scaleup_rank_idx = divmod(rank_idx, self.num_scaleup_ranks)
         self.num_rdma_ranks, self.num_nvlink_ranks = self.get_physical_domain_size()
         torch.cuda.synchronize()
 
     def destroy(self) -> None:
         super().destroy()
-        self.context = None
-        self.hccl_comm_handle = None
+        self.context = self.hccl_comm_handle = None
 
     @staticmethod
     def get_buffer_size_hint(group, num_max_tokens_per_rank: int, hidden: int, num_topk: int = 0,
@@ -188,27 +177,16 @@ class EPBuffer(BufferBase):
         return 0
 
     # ------------------------------------------------------------------------------------------
-    def dispatch(self,
-                 x: _TensorOrPair,
-                 topk_idx: Optional[torch.Tensor] = None,
+    def dispatch(self, x: _TensorOrPair, topk_idx: Optional[torch.Tensor] = None,
                  topk_weights: Optional[torch.Tensor] = None,
                  cumulative_local_expert_recv_stats: Optional[torch.Tensor] = None,
-                 num_experts: Optional[int] = None,
-                 num_max_tokens_per_rank: Optional[int] = None,
-                 expert_alignment: Optional[int] = None,
-                 num_sms: int = 0,
-                 num_qps: int = 0,
-                 previous_event: Optional[EventHandle] = None,
-                 async_with_compute_stream: bool = False,
-                 allocate_on_comm_stream: bool = False,
-                 handle: Optional[EPHandle] = None,
-                 do_handle_copy: bool = False,
-                 do_cpu_sync: Optional[bool] = None,
-                 do_expand: bool = False,
-                 do_zero_padding: bool = False,
-                 use_tma_aligned_col_major_sf: bool = False,
-                 defer_epilogue: bool = False,
-                 *, fused_fp8_quant: bool = False):
+                 num_experts: Optional[int] = None, num_max_tokens_per_rank: Optional[int] = None,
+                 expert_alignment: Optional[int] = None, num_sms: int = 0, num_qps: int = 0,
+                 previous_event: Optional[EventHandle] = None, async_with_compute_stream: bool = False,
+                 allocate_on_comm_stream: bool = False, handle: Optional[EPHandle] = None,
+                 do_handle_copy: bool = False, do_cpu_sync: Optional[bool] = None, do_expand: bool = False,
+                 do_zero_padding: bool = False, use_tma_aligned_col_major_sf: bool = False,
+                 defer_epilogue: bool = False, *, fused_fp8_quant: bool = False):
         """Send every token to the experts it selected.
 
         Arguments (as the reference, deep_ep/buffers/ep.py:340-375):
@@ -237,87 +215,84 @@ class EPBuffer(BufferBase):
         Returns `(recv_x or (recv_x, recv_sf), None, recv_topk_weights, handle, event)`, or the
         `EventOverlap` alone when `defer_epilogue`.
         """
-        if num_qps not in (None, 0):
-            raise NotImplementedError('Explicit QP counts are not implemented')
-        assert not do_handle_copy, '`do_handle_copy` must be False; handle copying is no longer supported'
-        x, sf = x if isinstance(x, tuple) else (x, None)
-        assert do_expand, 'only do_expand=True is supported'
+        self._no_explicit_qps(num_qps)
+        if do_handle_copy:
+            raise AssertionError('`do_handle_copy` must be False; handle copying is no longer supported')
+        if not do_expand:
+            raise AssertionError('only do_expand=True is supported')
+        payload, sf = x if isinstance(x, tuple) else (x, None)
 
-        cached = handle is not None
-        if cached:
-            assert topk_idx is None
-            assert handle.do_expand == do_expand
+        replay = handle is not None
+        if replay:
+            # the handle fixes the routing and every layout parameter; explicit values may only repeat them
+            assert topk_idx is None, 'a cached dispatch takes its routing from the handle'
             assert not do_cpu_sync, 'Cannot do CPU sync with cached handle'
-            topk_idx = handle.topk_idx
-            num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, handle.num_max_tokens_per_rank)
-            num_experts = value_or(num_experts, handle.num_experts)
-            expert_alignment = value_or(expert_alignment, handle.expert_alignment)
-            assert (num_experts, expert_alignment, num_max_tokens_per_rank) == \
-                   (handle.num_experts, handle.expert_alignment, handle.num_max_tokens_per_rank)
-            num_sms, do_cpu_sync = handle.num_sms, False
-            cached_fields = (handle.num_recv_tokens, handle.num_expanded_tokens,
-                             handle.num_recv_tokens_per_expert_list, handle.psum_num_recv_tokens_per_rank,
-                             handle.psum_num_recv_tokens_per_expert, handle.num_unaligned_recv_tokens_per_expert,
-                             handle.dst_buffer_slot_idx, handle.dst_gsge_idx, handle.recv_src_metadata)
+            assert handle.do_expand == do_expand
+            layout = (value_or(num_experts, handle.num_experts), value_or(expert_alignment, handle.expert_alignment),
+                      value_or(num_max_tokens_per_rank, handle.num_max_tokens_per_rank))
+            assert layout == (handle.num_experts, handle.expert_alignment, handle.num_max_tokens_per_rank)
+            num_experts, expert_alignment, num_max_tokens_per_rank = layout
+            topk_idx, num_sms, do_cpu_sync = handle.topk_idx, handle.num_sms, False
+            cached_fields = tuple(getattr(handle, name) for name in self._RUNTIME_CACHED_ORDER)
         else:
-            if num_sms == 0:
-                num_sms = self.get_theoretical_num_sms(num_experts, topk_idx.size(1))
-            cached_fields = (None,) * 9
-        num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, self.num_max_tokens_per_rank)
-        expert_alignment = value_or(expert_alignment, 1)
-        do_cpu_sync = value_or(do_cpu_sync, True)
+            num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, self.num_max_tokens_per_rank)
+            expert_alignment = value_or(expert_alignment, 1)
+            do_cpu_sync = value_or(do_cpu_sync, True)
+            num_sms = num_sms or self.get_theoretical_num_sms(num_experts, topk_idx.size(1))
+            cached_fields = (None,) * len(self._RUNTIME_CACHED_ORDER)
 
         result, event, deferred = self.runtime.dispatch(
-            x, sf, topk_idx, topk_weights, cumulative_local_expert_recv_stats, *cached_fields,
+            payload, sf, topk_idx, topk_weights, cumulative_local_expert_recv_stats, *cached_fields,
             num_max_tokens_per_rank, num_experts, expert_alignment, num_sms, previous_event,
             async_with_compute_stream, allocate_on_comm_stream, do_handle_copy, do_cpu_sync, do_expand,
             do_zero_padding, use_tma_aligned_col_major_sf, defer_epilogue, fused_fp8_quant=fused_fp8_quant)
         overlap = EventOverlap(event)
 
-        def finalize(res: tuple, sort_in_hook: bool):
-            (recv_x, recv_sf, recv_topk_weights, num_recv_tokens, num_expanded_tokens, per_expert_list,
-             psum_rank, psum_expert, unaligned, recv_src_metadata, dst_slot, dst_gsge) = res
-            nonlocal handle
-            if not cached:
-                handle = EPHandle(do_expand, num_experts, expert_alignment, num_max_tokens_per_rank, num_sms,
-                                  topk_idx, num_recv_tokens, num_expanded_tokens, per_expert_list, psum_rank,
-                                  psum_expert, unaligned, recv_src_metadata, dst_slot, dst_gsge)
+        def finish(native_result: tuple, sort_when_waited: bool):
+            recv_x, recv_sf, recv_topk_weights, *layout_fields = native_result
+            this_handle = handle if replay else EPHandle(do_expand, num_experts, expert_alignment,
+                                                         num_max_tokens_per_rank, num_sms, topk_idx, *layout_fields)
             if self.deterministic:
-                def canonicalise():
-                    handle.deterministic_sort(do_cpu_sync, cached, recv_x, recv_sf, recv_topk_weights)
-                if sort_in_hook:
-                    overlap.register_hook_after_wait(canonicalise)
+                def canonical_order():
+                    this_handle.deterministic_sort(do_cpu_sync, replay, recv_x, recv_sf, recv_topk_weights)
+                if sort_when_waited:
+                    overlap.register_hook_after_wait(canonical_order)
                 else:
-                    canonicalise()
-            return (recv_x, recv_sf) if recv_sf is not None else recv_x, None, recv_topk_weights, handle
+                    canonical_order()
+            received = recv_x if recv_sf is None else (recv_x, recv_sf)
+            return received, None, recv_topk_weights, this_handle
 
-        if deferred is not None:
-            overlap.register_hook_after_wait(lambda: finalize(deferred(), False))
-            return overlap
-        assert result is not None
-        return (*finalize(result, async_with_compute_stream), overlap)
+        if deferred is None:
+            return (*finish(result, async_with_compute_stream), overlap)
+        overlap.register_hook_after_wait(lambda: finish(deferred(), False))
+        return overlap
+
+    # order in which the native runtime takes the fields of a cached handle (csrc/buffers/ep.hpp:96-104)
+    _RUNTIME_CACHED_ORDER = ('num_recv_tokens', 'num_expanded_tokens', 'num_recv_tokens_per_expert_list',
+                             'psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
+                             'num_unaligned_recv_tokens_per_expert', 'dst_buffer_slot_idx', 'dst_gsge_idx',
+                             'recv_src_metadata')
+
+    @staticmethod
+    def _no_explicit_qps(num_qps) -> None:
+        if num_qps:
+            raise NotImplementedError('Explicit QP counts are not implemented')
 
     @staticmethod
     def _unpack_bias(bias) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-        if isinstance(bias, torch.Tensor):
+        """None, one tensor, or a pair -> always a pair."""
+        if bias is None:
+            return None, None
+        if torch.is_tensor(bias):
             return bias, None
-        if isinstance(bias, tuple):
-            assert len(bias) == 2
-            return bias
-        return None, None
+        first, second = bias
+        return first, second
 
-    def combine(self,
-                x: torch.Tensor,
-                handle: EPHandle,
-                topk_weights: Optional[torch.Tensor] = None,
-                bias: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]] = None,
-                num_sms: int = 0,
-                num_qps: int = 0,
-                previous_event: EventHandle = None,
-                async_with_compute_stream: bool = False,
-                allocate_on_comm_stream: bool = False,
-                defer_epilogue: bool = False,
-                *, apply_weights: bool = False):
+    def combine(self, x: torch.Tensor, handle: EPHandle, topk_weights: Optional[torch.Tensor] = None,
+                bias: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]] = None, num_sms: int = 0,
+                num_qps: int = 0, previous_event: EventHandle = None, async_with_compute_stream: bool = False,
+                allocate_on_comm_stream: bool = False, defer_epilogue: bool = False, *,
+                apply_weights: bool = False):
         """Reduce expert outputs back to token order.
 
         Arguments (as the reference, deep_ep/buffers/ep.py:536-550):
@@ -333,9 +308,9 @@ class EPBuffer(BufferBase):
 
         Returns `(combined_x, combined_topk_weights, event)`, or the `EventOverlap` alone.
         """
-        if num_qps not in (None, 0):
-            raise NotImplementedError('Explicit QP counts are not implemented')
-        assert handle.recv_src_metadata is not None
+        self._no_explicit_qps(num_qps)
+        if handle.recv_src_metadata is None:
+            raise AssertionError('the handle comes from a dispatch that ran its epilogue')
         bias_0, bias_1 = self._unpack_bias(bias)
         result, event, deferred = self.runtime.combine(
             x, topk_weights, bias_0, bias_1, handle.recv_src_metadata, handle.topk_idx,
@@ -343,11 +318,10 @@ class EPBuffer(BufferBase):
             handle.num_sms, previous_event, async_with_compute_stream, allocate_on_comm_stream, defer_epilogue,
             apply_weights=apply_weights)
         overlap = EventOverlap(event)
-        if deferred is not None:
-            overlap.register_hook_after_wait(deferred)
-            return overlap
-        assert result is not None
-        return (*result, overlap)
+        if deferred is None:
+            return (*result, overlap)
+        overlap.register_hook_after_wait(deferred)
+        return overlap
 
     # ---- load-balancing entry points: storage exists, kernels do not (csrc/buffers/ep.hpp:75-86) ----
     def lb_get_theoretical_num_sms(self) -> int:
