@@ -182,3 +182,82 @@ def test_c5_one_gpu_share_of_ep32():
     for (grp, src), p in own_p.items():
         assert torch.equal(P[grp, src - rank * T].cpu().view(torch.int16), p.view(torch.int16))
     buf.destroy()
+
+
+def test_ep32_node_full_size_properties():
+    """The EP32 configuration with all 32 partitions on the GPU, each dispatching the full 16384 x 7168
+    tokens (fused FP8) with a routing of its own: every partition receives its real share from 32 sources.
+    Checked through properties that hold at any size: per-source counts, the received rows are the
+    quantised source tokens bit for bit, slots tile the experts' aligned blocks, padding is zero, and the
+    combine returns (number of selections) x (a small-integer row), exactly."""
+    import deep_ep
+    R, T, H, E, K, A = 32, 16384, 7168, 256, 6, 128
+    El = E // R
+    node = deep_ep.LocalNode(R)
+    bufs = [deep_ep.EPBuffer(node.group(r), num_max_tokens_per_rank=T, hidden=H, num_topk=K, use_fp8_dispatch=True,
+                             explicitly_destroy=True) for r in range(R)]
+    x = make_tokens(T, H, seed=0, outliers=True)
+    q, s = O.quantise(x)                                         # CPU quantiser = the reference's arithmetic
+    qg, sg, xg = q.to(DEV), s.to(DEV), x.to(DEV)
+    base_topk, base_w = make_routing(T, E, K, seed=0, masked=0.05)
+    # partition r routes token t like the base routing of token (t + 97 r) mod T, experts rotated by r
+    topks, wts = [], []
+    for r in range(R):
+        t_ = torch.roll(base_topk, shifts=-97 * r, dims=0)
+        topks.append(torch.where(t_ >= 0, (t_ + r) % E, t_).to(DEV))
+        wts.append(torch.roll(base_w, shifts=-97 * r, dims=0).to(DEV))
+
+    events = [bufs[r].dispatch(xg, topk_idx=topks[r], topk_weights=wts[r], num_experts=E, num_max_tokens_per_rank=T,
+                               expert_alignment=A, do_expand=True, do_zero_padding=True, fused_fp8_quant=True,
+                               async_with_compute_stream=True, defer_epilogue=True) for r in range(R)]
+    z = (torch.arange(T, device=DEV).view(T, 1) * 3 + torch.arange(H, device=DEV).view(1, H)) % 7 - 3
+    z = z.to(torch.bfloat16)                                      # "expert output" of a token: small integers
+    handles, partial_events = [], []
+    all_topk = torch.stack(topks)                                 # [R, T, K]
+    for d in range(R):
+        (rx, rsf), _, rw, handle = events[d].current_stream_wait()
+        meta = handle.recv_src_metadata.long()
+        slots, src = meta[:, :K], meta[:, K]
+        src_rank, src_tok = src // T, src % T
+        # per source: exactly its tokens with a selection on partition d, in token order
+        psum = [0] + handle.psum_num_recv_tokens_per_rank.tolist()
+        local_any = ((all_topk >= d * El) & (all_topk < (d + 1) * El)).any(dim=2)     # [R, T]
+        assert psum[1:] == torch.cumsum(local_any.sum(dim=1), 0).tolist()
+        for sr in (0, d, R - 1):
+            part = slice(psum[sr], psum[sr + 1])
+            assert torch.equal(src_tok[part], local_any[sr].nonzero().flatten())
+            assert bool((src_rank[part] == sr).all())
+        sel = all_topk[src_rank, src_tok]                           # [N, K] global expert ids
+        local = (sel >= d * El) & (sel < (d + 1) * El)
+        assert torch.equal(slots >= 0, local)
+        flat = slots[local]
+        assert torch.unique(flat).numel() == flat.numel() == int(handle.num_unaligned_recv_tokens_per_expert.sum())
+        tok_of_slot = src_tok.unsqueeze(1).expand(-1, K)[local]
+        assert torch.equal(rx.view(torch.uint8)[flat], qg[tok_of_slot])
+        assert torch.equal(rsf[flat], sg[tok_of_slot])
+        assert torch.equal(rw[flat], torch.stack(wts)[src_rank, src_tok][local])
+        pad = torch.ones(rx.size(0), dtype=torch.bool, device=DEV)
+        pad[flat] = False
+        assert int(rx.view(torch.uint8)[pad].count_nonzero()) == 0 and int(rsf[pad].count_nonzero()) == 0
+        cnt = handle.num_unaligned_recv_tokens_per_expert.long()
+        start = handle.psum_num_recv_tokens_per_expert.long() - cnt
+        assert bool((start % A == 0).all())
+        assert torch.equal(cnt, torch.bincount(sel[local] - d * El, minlength=El))
+        # experts are the identity on z: row of (source token, j) = z[token]
+        y = torch.full((rx.size(0), H), 99.0, dtype=torch.bfloat16, device=DEV)
+        y[flat] = z[tok_of_slot]
+        handles.append((handle, y, rw))
+        del rx, rsf
+    # every partition has expanded what it received: only now may the combine reuse the buffers
+    for d, (handle, y, rw) in enumerate(handles):
+        partial_events.append(bufs[d].combine(y, handle, topk_weights=rw, async_with_compute_stream=True,
+                                              defer_epilogue=True))
+    del handles
+    for r in range(R):
+        cx, cw = partial_events[r].current_stream_wait()
+        n_sel = (topks[r] >= 0).sum(dim=1, keepdim=True).to(torch.float32)
+        assert torch.equal(cx.float(), z.float() * n_sel), r      # small integers: every sum and rounding is exact
+        assert torch.equal(cw, wts[r])
+    torch.cuda.synchronize()
+    for b in bufs:
+        b.destroy()
