@@ -362,6 +362,8 @@ class EPBuffer(BufferBase):
                  do_expand, do_zero_padding, use_col_major_sf, defer_epilogue, fused_fp8_quant=False):
         if self.destroyed:
             raise EPException('Assertion exception (_C.py): not destroyed')
+        if previous_event is not None:
+            previous_event.current_stream_wait()       # the launches below are ordered behind it
         if not do_expand:
             raise EPException('Assertion exception (_C.py): do_expand')
         if do_handle_copy:
@@ -535,6 +537,8 @@ class EPBuffer(BufferBase):
                 async_with_compute_stream, allocate_on_comm_stream, defer_epilogue, apply_weights=False):
         if self.destroyed:
             raise EPException('Assertion exception (_C.py): not destroyed')
+        if previous_event is not None:
+            previous_event.current_stream_wait()
         if num_sms <= 0:
             raise EPException('Assertion exception (_C.py): num_sms > 0')
         if x.dim() != 2 or combined_topk_idx.dim() != 2:

@@ -198,7 +198,8 @@ class EPBuffer(BufferBase):
             num_experts, num_max_tokens_per_rank, expert_alignment: layout parameters (taken
                 from the handle when one is given; alignment defaults to 1).
             num_sms: recorded in the handle; launches size themselves.  num_qps must be 0.
-            previous_event, allocate_on_comm_stream: accepted and ignored.
+            previous_event: an `EventHandle` the current stream waits for before anything is enqueued.
+            allocate_on_comm_stream: accepted and ignored (there is one stream).
             async_with_compute_stream: also return an event for the enqueued work.
             handle: a previous `EPHandle` to replay (no layout pass, no host sync).
             do_cpu_sync: read exact counts on the host before allocating outputs (default True

@@ -246,3 +246,30 @@ def test_plain_c_caller_of_the_abi():
     res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert res.returncode == 0, res.stderr
     assert res.stdout.startswith('abi_client: ok')
+
+
+def test_previous_event_orders_the_dispatch_behind_another_stream():
+    """The inputs are produced on a side stream; `previous_event` (captured there) is all that orders the
+    dispatch on the current stream behind them."""
+    import deep_ep
+    T, H, E, K = 2048, 2048, 16, 4
+    buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K, explicitly_destroy=True)
+    topk, w = make_routing(T, E, K, seed=3)
+    tg, wg = topk.to(DEV), w.to(DEV)
+    src = make_tokens(T, H, seed=3).to(DEV)
+    x = torch.zeros_like(src)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(20):                       # keep the side stream busy before the inputs appear
+            junk = torch.randn((2048, 2048), device=DEV) @ torch.randn((2048, 2048), device=DEV)
+        x.copy_(src)
+        ready = deep_ep.EPBuffer.capture()
+    rx, _, _, handle, _ = buf.dispatch(x, topk_idx=tg, topk_weights=wg, num_experts=E, do_expand=True,
+                                       previous_event=ready)
+    torch.cuda.synchronize()
+    del junk
+    meta = handle.recv_src_metadata.long()
+    valid = meta[:, :K] >= 0
+    assert torch.equal(rx[meta[:, :K][valid]], src[meta[:, K]].unsqueeze(1).expand(-1, K, -1)[valid])
+    buf.destroy()
