@@ -51,8 +51,8 @@ __device__ __forceinline__ int wave_inclusive_sum(int v) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Layout pass A: per-block histograms of expert ids and of destination-partition masters.
-// Reference semantics: impls/ep/dispatch.hpp:166-194 (expert histogram, dedup by partition).
+// Entries of the layout passes: (token, j) of topk_idx on the send side, (row, j) of the receive
+// stream on the receive side.
 // ------------------------------------------------------------------------------------------------
 // Receive side: inclusive row counts per source partition from the inbox, in LDS.  Every thread of
 // the workgroup calls it (blockDim >= R); returns the length of the receive stream.  s_psum holds
@@ -130,6 +130,10 @@ __device__ __forceinline__ int master_rank(const short* s_rk, int idx, int K) {
     return r;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Layout pass A: per-block histograms of expert ids and of destination-partition masters.
+// Reference semantics: impls/ep/dispatch.hpp:166-194 (expert histogram, dedup by partition).
+// ------------------------------------------------------------------------------------------------
 extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(EpLayoutArgs a) {
     extern __shared__ int smem[];
     const int E = a.num_experts, R = a.num_ranks, K = a.num_topk;
@@ -601,8 +605,8 @@ __device__ __forceinline__ void zero_padding_rows(const EpScatterArgs& a) {
     const int e = pb / a.pad_blocks_per_expert, part = pb % a.pad_blocks_per_expert;
     if (e >= a.num_local_experts) return;
     const int end = a.psum_expert[e];
-    const int rows = align_up(end, a.expert_alignment) - end;
-    if (rows <= 0) return;
+    const int rows = min(align_up(end, a.expert_alignment), a.num_out_rows) - end;     // never past the outputs
+    if (end < 0 || rows <= 0) return;
     zero_span((char*)a.recv_x + (int64_t)end * a.out_row_bytes, (int64_t)rows * a.out_row_bytes, part,
               a.pad_blocks_per_expert);
     if (a.recv_sf != nullptr && part == 0)

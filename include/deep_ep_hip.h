@@ -11,6 +11,10 @@
  *   - all device pointers belong to the device that was current when the buffer was created;
  *     all kernels are enqueued on the `stream` argument and nothing synchronises unless said.
  *   - an ep_tensor_t with data == NULL means "absent".
+ *   - a buffer is driven by one host thread at a time; different buffers may be used from
+ *     different threads (ep_last_error is per thread).
+ *   - none of the launch functions allocates, frees, memsets or synchronises: they only validate
+ *     and enqueue kernels, so they can be recorded into a HIP graph.
  */
 #ifndef DEEP_EP_HIP_H
 #define DEEP_EP_HIP_H
