@@ -295,3 +295,60 @@ def test_node_with_an_empty_partition_and_disconnect():
     lay = O.rank_share_layout(topks[0].numpy(), E, R, 0, A, max_tokens)
     assert np.array_equal(handle.recv_src_metadata.cpu().numpy(), lay['recv_src_metadata'])
     bufs[0].destroy()
+
+
+def test_node_hand_derived_two_rank_example():
+    """A case small enough to derive by hand from the reference's code: R=2, E=4, K=2, A=2, maxT=4; rank 0
+    holds three tokens with topk_idx [[0,1],[3,-1],[2,0]], rank 1 holds none.  Expected values are written
+    out literally, not computed by the oracle."""
+    R, max_tokens, H, E, K, A = 2, 4, 64, 4, 2, 2
+    bufs = make_node(R, max_tokens, H, K, False)
+    x0 = make_tokens(3, H, seed=5)
+    topk0 = torch.tensor([[0, 1], [3, -1], [2, 0]], dtype=torch.int64)
+    w0 = torch.tensor([[0.25, 0.75], [1.0, 0.0], [0.5, 0.5]], dtype=torch.float32)
+    xs = [x0, torch.empty((0, H), dtype=torch.bfloat16)]
+    topks = [topk0, torch.empty((0, K), dtype=torch.int64)]
+    ws = [w0, torch.empty((0, K), dtype=torch.float32)]
+    outs = dispatch_all(bufs, [x.to(DEV) for x in xs], [t.to(DEV) for t in topks], [w.to(DEV) for w in ws],
+                        num_experts=E, num_max_tokens_per_rank=max_tokens, expert_alignment=A, do_expand=True,
+                        do_zero_padding=True)
+    torch.cuda.synchronize()
+    (rx0, _, rw0, h0), (rx1, _, rw1, h1) = outs
+    zero = torch.zeros(H, dtype=torch.bfloat16)
+    # rank 0: receives t0 (experts 0 and 1) and t2 (expert 0 at j=1)
+    assert h0.dst_buffer_slot_idx.tolist() == [[-1, 0], [0, -1], [1, 1]]
+    assert h0.psum_num_recv_tokens_per_rank.tolist() == [2, 2]
+    assert h0.num_unaligned_recv_tokens_per_expert.tolist() == [2, 1]
+    assert h0.psum_num_recv_tokens_per_expert.tolist() == [2, 3]
+    assert (h0.num_recv_tokens, h0.num_expanded_tokens, h0.num_recv_tokens_per_expert_list) == (2, 4, [2, 2])
+    assert h0.recv_src_metadata.tolist() == [[0, 2, 0, 1], [-1, 1, 2, 1]]
+    assert torch.equal(rx0.cpu(), torch.stack([x0[0], x0[2], x0[0], zero]))
+    assert rw0.tolist() == [0.25, 0.5, 0.75, 0.0]
+    # rank 1: receives t1 (expert 3 = local 1) and t2 (expert 2 = local 0)
+    assert h1.psum_num_recv_tokens_per_rank.tolist() == [2, 2]
+    assert h1.num_unaligned_recv_tokens_per_expert.tolist() == [1, 1]
+    assert h1.psum_num_recv_tokens_per_expert.tolist() == [1, 3]
+    assert h1.recv_src_metadata.tolist() == [[2, -1, 1, 0], [0, -1, 2, 0]]
+    assert torch.equal(rx1.cpu(), torch.stack([x0[2], zero, x0[1], zero]))
+    assert rw1.tolist() == [0.5, 0.0, 1.0, 0.0]
+
+    g = torch.Generator().manual_seed(1)
+    y0 = torch.randn((4, H), generator=g).to(torch.bfloat16)
+    y1 = torch.randn((4, H), generator=g).to(torch.bfloat16)
+    b0 = torch.randn((3, H), generator=g).to(torch.bfloat16)
+    b1 = torch.randn((3, H), generator=g).to(torch.bfloat16)
+    empty_bias = tuple(torch.empty((0, H), dtype=torch.bfloat16, device=DEV) for _ in range(2))
+    res = combine_all(bufs, [y0.to(DEV), y1.to(DEV)], [h0, h1], [rw0, rw1], [(b0.to(DEV), b1.to(DEV)), empty_bias])
+    torch.cuda.synchronize()
+    cx, cw = res[0]
+    p_t0 = (y0[0].float() + y0[2].float()).to(torch.bfloat16)           # owner 0, two local slots
+    bias = b0.float() + b1.float()
+    want = torch.stack([
+        (bias[0] + p_t0.float()).to(torch.bfloat16),
+        (bias[1] + y1[2].float()).to(torch.bfloat16),                       # t1: one master, partial = y1[2] verbatim
+        (bias[2] + y1[0].float() + y0[1].float()).to(torch.bfloat16),       # t2: masters j=0 (rank 1) then j=1 (rank 0)
+    ])
+    assert torch.equal(cx.cpu().view(torch.int16), want.view(torch.int16))
+    assert torch.equal(cw.cpu(), w0)
+    for b in bufs:
+        b.destroy()
