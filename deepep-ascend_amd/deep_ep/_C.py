@@ -10,7 +10,7 @@ module raises.
 """
 import ctypes
 import os
-from typing import Callable, List, Optional, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import bf16_bits, bf16_from_bits, make_routing, make_tokens
+from helpers import bf16_bits, make_routing, make_tokens
 from oracle import ep_oracle as O
 
 pytestmark = pytest.mark.gpu

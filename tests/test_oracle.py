@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import bf16_bits, bf16_from_bits, make_routing, make_tokens
+from helpers import bf16_from_bits, make_routing, make_tokens
 from oracle import ep_oracle as O
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden')
