@@ -163,3 +163,18 @@ int main(void) {
            ctypes.sizeof(C._DispatchRecvArgs), C._DispatchRecvArgs.stream.offset,
            C._DispatchRecvArgs.hidden_bytes.offset]
     assert got == [int(v) for v in out]
+
+
+def test_bench_byte_formulas_give_the_headline_figures():
+    """The algorithmic bytes bench.py prices the kernels with, at the headline configuration
+    (16384 x 7168, top-6, every selection valid): 14 336 B read + 6 x 7396 B written per token plus
+    metadata for the fused FP8 dispatch, 6 x 14 336 B read + 14 336 B written for the combine."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location('bench_module', os.path.join(ROOT, 'bench.py'))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    T, H, K = 16384, 7168, 6
+    assert bench.dispatch_bytes(T, H, K, T * K, T, True, True) == 964427776
+    assert bench.combine_bytes(T, H, K, T * K, T, 0, True) == 1646264320
+    assert bench.dispatch_bytes(4096, H, 8, 4096 * 8, 4096, False, False) == 529432576      # BF16 top-8
+    assert bench.WORKLOADS['c3_headline'] == (T, H, 256, K, 128, True)
