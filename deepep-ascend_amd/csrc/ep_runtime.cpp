@@ -391,6 +391,27 @@ int ep_buffer_connect(ep_buffer_t** bufs, int n) {
     });
 }
 
+int ep_buffer_set_peers(ep_buffer_t* b, void* const* arena_bases, int n) {
+    return guarded([&] {
+        check_buffer(b);
+        HIP_CHECK(hipDeviceSynchronize());
+        if (arena_bases == nullptr) {
+            disconnect(b);
+            return;
+        }
+        EP_HOST_ASSERT(n == b->num_ranks and n > 1);
+        std::vector<char*> arenas(n);
+        for (int i = 0; i < n; ++i) {
+            EP_HOST_ASSERT(arena_bases[i] != nullptr);
+            arenas[i] = (char*)arena_bases[i];
+        }
+        EP_HOST_ASSERT(arenas[b->rank_idx] == b->arena and "a partition's own entry is its own arena");
+        write_peer_table(b, arenas);
+        b->connected = true;
+        b->peers.clear();           // arenas the caller mapped: theirs to keep alive and to disconnect
+    });
+}
+
 int ep_buffer_destroy(ep_buffer_t* b) {
     return guarded([&] {
         EP_HOST_ASSERT(b != nullptr);

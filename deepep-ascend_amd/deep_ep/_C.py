@@ -99,6 +99,7 @@ _ep_worst = _sig('ep_dispatch_worst_case_sizes', ctypes.c_int, ctypes.c_void_p, 
                  ctypes.c_int, ctypes.c_int, _c_int_p, _c_int_p)
 _ep_dispatch_recv = _sig('ep_dispatch_recv_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_DispatchRecvArgs))
 _ep_connect = _sig('ep_buffer_connect', ctypes.c_int, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int)
+_ep_set_peers = _sig('ep_buffer_set_peers', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int)
 _ep_dispatch_epi = _sig('ep_dispatch_epilogue_launch', ctypes.c_int, ctypes.c_void_p,
                         ctypes.POINTER(_DispatchEpilogueArgs))
 _ep_combine = _sig('ep_combine_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_CombineArgs), ctypes.c_int)
@@ -323,6 +324,17 @@ class EPBuffer(BufferBase):
 
     def print_memory_usage(self) -> None:
         _check(_ep_print_mem(self._h))
+
+    def set_peers(self, arena_bases) -> None:
+        """Connects this partition alone, by address: `arena_bases[i]` is where partition i's arena (its
+        `region(0)` pointer) is mapped in this process; None disconnects."""
+        if arena_bases is None:
+            _check(_ep_set_peers(self._h, None, 0))
+            self.connected = False
+            return
+        table = (ctypes.c_void_p * len(arena_bases))(*arena_bases)
+        _check(_ep_set_peers(self._h, table, len(arena_bases)))
+        self.connected = True
 
     @staticmethod
     def connect(runtimes) -> None:

@@ -100,6 +100,14 @@ int ep_buffer_create(int rank_idx, int num_ranks, int64_t num_bytes, int64_t num
  * partition disconnects the others.  Synchronises.  No counterpart call in the reference, whose
  * ranks find each other through the process group. */
 int ep_buffer_connect(ep_buffer_t** bufs, int n);
+/* The same connection, one partition at a time and by address: arena_bases[i] is where partition i's
+ * arena (what ep_buffer_region(peer, 0, ..) returns in the process that owns it) can be reached from
+ * this process -- the pointer itself for a buffer of this process, or the mapping of that
+ * allocation obtained otherwise (hipIpcOpenMemHandle in a process per GPU).  arena_bases[rank] must
+ * be this buffer's own arena; all arenas must have been created with the same sizes.  The caller
+ * keeps the mappings alive while the buffer is connected; arena_bases == NULL disconnects.
+ * Synchronises. */
+int ep_buffer_set_peers(ep_buffer_t* buf, void* const* arena_bases, int n);
 /* EPBuffer::destroy (csrc/buffers/ep.hpp:65-73). */
 int ep_buffer_destroy(ep_buffer_t* buf);
 /* which: 0 workspace, 1 buffer, 2 lb storage (csrc/buffers/ep.hpp:50-53). */

@@ -352,3 +352,46 @@ def test_node_hand_derived_two_rank_example():
     assert torch.equal(cw.cpu(), w0)
     for b in bufs:
         b.destroy()
+
+
+def test_partitions_connected_by_address():
+    """ep_buffer_set_peers: the connection a process per GPU would make with mapped arena addresses, here
+    with the addresses of three buffers of this process; same results as a node."""
+    import deep_ep
+    R, max_tokens, H, E, K, A = 3, 50, 128, 6, 3, 4
+    bufs = [deep_ep.EPBuffer(deep_ep.LocalGroup(r, R), num_max_tokens_per_rank=max_tokens, hidden=H, num_topk=K,
+                             explicitly_destroy=True) for r in range(R)]
+    bases = [b.runtime.region(0)[0] for b in bufs]
+    for b in bufs:
+        b.runtime.set_peers(bases)
+    Ts = [50, 41, 17]
+    xs = [make_tokens(T, H, seed=60 + r) for r, T in enumerate(Ts)]
+    routing = [make_routing(T, E, K, seed=70 + r, masked=0.1) for r, T in enumerate(Ts)]
+    topks, ws = [t for t, _ in routing], [w for _, w in routing]
+    rows = [bf16_bits(x).view(np.uint8).reshape(x.size(0), H * 2) for x in xs]
+    _, want = oracle_dispatch(rows, [None] * R, [t.numpy() for t in topks], [w.numpy() for w in ws], E, R, A, max_tokens)
+    outs = dispatch_all(bufs, [x.to(DEV) for x in xs], [t.to(DEV) for t in topks], [w.to(DEV) for w in ws],
+                        num_experts=E, num_max_tokens_per_rank=max_tokens, expert_alignment=A, do_expand=True,
+                        do_zero_padding=True)
+    torch.cuda.synchronize()
+    for r, (rx, _, rw, handle) in enumerate(outs):
+        assert np.array_equal(handle.recv_src_metadata.cpu().numpy(), want[r]['lay']['recv_src_metadata'])
+        assert np.array_equal(rx.view(torch.uint8).cpu().numpy().reshape(rx.size(0), H * 2), want[r]['x'])
+    res = combine_all(bufs, [o[0] for o in outs], [o[3] for o in outs], [o[2] for o in outs], [None] * R)
+    torch.cuda.synchronize()
+    for r in range(R):
+        n_sel = (topks[r] >= 0).sum(dim=1, keepdim=True)
+        # identity experts: every partial is a sum of copies of the token; compare with the oracle's two-level sum
+        parts, wv = {}, {}
+        for d in range(R):
+            p, w_ = O.combine_partial(torch.from_numpy(want[d]['x'].view(np.int16)).view(torch.bfloat16),
+                                      torch.from_numpy(want[d]['w']), want[d]['lay']['recv_src_metadata'], R, d, max_tokens)
+            parts.update(p)
+            wv.update(w_)
+        ox, ow = O.combine_final(topks[r].numpy(), E, R, r, max_tokens, lambda k: parts[k], lambda k: wv[k],
+                                 None, None, H, True)
+        assert np.array_equal(bf16_bits(res[r][0]), bf16_bits(ox)) and n_sel.numel() == Ts[r]
+        assert torch.equal(res[r][1].cpu(), ow)
+    for b in bufs:
+        b.runtime.set_peers(None)
+        b.destroy()
