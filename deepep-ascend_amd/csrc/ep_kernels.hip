@@ -436,14 +436,16 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
 __device__ __forceinline__ float bf16_lo(unsigned int u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(unsigned int u) { return __uint_as_float(u & 0xffff0000u); }
 
-// max over the 16 lanes of a DPP row, result in every lane of the row
-__device__ __forceinline__ float row16_max(float v) {
-    int x = __float_as_int(v);
-    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x128, 0xf, 0xf, false))));  // row_ror:8
-    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x124, 0xf, 0xf, false))));  // row_ror:4
-    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x122, 0xf, 0xf, false))));  // row_ror:2
-    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x121, 0xf, 0xf, false))));  // row_ror:1
-    return __int_as_float(x);
+// Largest magnitude over the 16 lanes of a DPP row, result in every lane of the row.  The operands
+// are the bit patterns of |x|: as unsigned integers they order like the floats, +inf above every
+// finite value and NaN above +inf, so a NaN anywhere in the group comes out as the group's maximum,
+// as it does from torch's amax (deep_ep/utils/math.py:36).
+__device__ __forceinline__ unsigned row16_umax(unsigned x) {
+    x = max(x, (unsigned)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x128, 0xf, 0xf, false));  // row_ror:8
+    x = max(x, (unsigned)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x124, 0xf, 0xf, false));  // row_ror:4
+    x = max(x, (unsigned)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x122, 0xf, 0xf, false));  // row_ror:2
+    x = max(x, (unsigned)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x121, 0xf, 0xf, false));  // row_ror:1
+    return x;
 }
 
 template <bool HW>
@@ -698,14 +700,15 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     if (live) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
     float f[8] = {bf16_lo(d.x), bf16_hi(d.x), bf16_lo(d.y), bf16_hi(d.y),
                   bf16_lo(d.z), bf16_hi(d.z), bf16_lo(d.w), bf16_hi(d.w)};
-    float m = 0.0f;
+    unsigned mbits = 0u;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) m = fmaxf(m, fabsf(f[q]));
-    m = row16_max(m);
-    const float amax = fmaxf(m, 1e-4f);
+    for (int q = 0; q < 8; ++q) mbits = max(mbits, __float_as_uint(f[q]) & 0x7fffffffu);
+    const float m = __uint_as_float(row16_umax(mbits));
+    const float amax = m < 1e-4f ? 1e-4f : m;       // clamp(min=1e-4): a NaN stays a NaN
     const float inv = (1.0f / amax) * 448.0f;       // torch evaluates `448.0 / t` as t.reciprocal() * 448.0
     const float scale = amax / 448.0f;
-    const u32x2 q8 = quant8<HW>(f, inv);
+    u32x2 q8 = quant8<HW>(f, inv);
+    if (amax != amax) q8 = u32x2{0x7f7f7f7fu, 0x7f7f7f7fu};   // every product is NaN: e4m3fn has one NaN, sign clear
     if (!live) return;
     const bool writes_scale = (lane & 15) == 0;
     for (int j = 0; j < K; ++j) {

@@ -273,3 +273,31 @@ def test_previous_event_orders_the_dispatch_behind_another_stream():
     valid = meta[:, :K] >= 0
     assert torch.equal(rx[meta[:, :K][valid]], src[meta[:, K]].unsqueeze(1).expand(-1, K, -1)[valid])
     buf.destroy()
+
+
+@pytest.mark.parametrize('hw_convert', [True, False])
+def test_fused_quantiser_on_non_finite_inputs(hw_convert):
+    """inf, -inf, NaN, -NaN, an all-zero row and the largest BF16 go through the fused quantiser exactly as
+    through the reference's arithmetic (deep_ep/utils/math.py:30-38: amax and clamp propagate a NaN to the
+    whole 128-channel group and its scale; an infinity makes the multiplier zero)."""
+    import deep_ep
+    T, H, E, K = 8, 256, 4, 1
+    x = make_tokens(T, H, seed=12)
+    x[0, 3], x[1, 5], x[2, 7], x[5, 130] = float('inf'), float('-inf'), float('nan'), -float('nan')
+    x[3, :] = 0
+    x[4, 0] = 3.3e38
+    topk = torch.zeros((T, K), dtype=torch.int64)
+    q, s = O.quantise(x)
+    buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K, use_fp8_dispatch=True,
+                           explicitly_destroy=True)
+    deep_ep._C.set_fp8_hw_convert(hw_convert)
+    try:
+        (rx, rsf), _, _, _, _ = buf.dispatch(x.to(DEV), topk_idx=topk.to(DEV), num_experts=E, do_expand=True,
+                                             fused_fp8_quant=True)
+        torch.cuda.synchronize()
+    finally:
+        deep_ep._C.set_fp8_hw_convert(True)
+    assert np.array_equal(rx.view(torch.uint8).cpu().numpy(), q.numpy())
+    assert np.array_equal(rsf.cpu().numpy().view(np.uint32), s.numpy().view(np.uint32))
+    assert int((q.numpy()[2, :128] == 0x7f).sum()) == 128          # the NaN poisons its whole group
+    buf.destroy()
