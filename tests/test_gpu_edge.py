@@ -301,3 +301,33 @@ def test_fused_quantiser_on_non_finite_inputs(hw_convert):
     assert np.array_equal(rsf.cpu().numpy().view(np.uint32), s.numpy().view(np.uint32))
     assert int((q.numpy()[2, :128] == 0x7f).sum()) == 128          # the NaN poisons its whole group
     buf.destroy()
+
+
+def test_combine_on_non_finite_expert_outputs():
+    """inf, -inf (their sum: NaN) and NaN rows go through the fp32 accumulation and the single rounding as in
+    the reference's ordered sum (deep_ep/utils/refs.py:155-173)."""
+    import deep_ep
+    T, H, E, K, A = 40, 128, 4, 3, 2
+    x = make_tokens(T, H, seed=21)
+    topk, w = make_routing(T, E, K, seed=21, masked=0.2)
+    lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, T)
+    buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K, explicitly_destroy=True)
+    _, _, rw, handle, _ = buf.dispatch(x.to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV), num_experts=E,
+                                       expert_alignment=A, do_expand=True, do_zero_padding=True)
+    g = torch.Generator().manual_seed(2)
+    y = torch.randn((lay['num_expanded_tokens'], H), generator=g).to(torch.bfloat16)
+    r = torch.rand(y.shape, generator=g)
+    y[r < 0.02] = float('inf')
+    y[(r >= 0.02) & (r < 0.04)] = float('-inf')
+    y[(r >= 0.04) & (r < 0.05)] = float('nan')
+    y[(r >= 0.05) & (r < 0.06)] = 3.3e38                     # sums overflow to inf
+    bias = torch.randn((T, H), generator=g).to(torch.bfloat16)
+    for b in (None, bias):
+        cx, _, _ = buf.combine(y.to(DEV), handle, topk_weights=rw, bias=None if b is None else b.to(DEV))
+        torch.cuda.synchronize()
+        ox, _ = O.combine_fast(y, None, lay['recv_src_metadata'], T, K, b)
+        got, want = bf16_bits(cx), bf16_bits(ox)
+        both_nan = ((got & 0x7fff) > 0x7f80) & ((want & 0x7fff) > 0x7f80)      # any NaN equals any NaN
+        assert ((got == want) | both_nan).all()
+        assert both_nan.any() and ((want & 0x7fff) == 0x7f80).any()
+    buf.destroy()
