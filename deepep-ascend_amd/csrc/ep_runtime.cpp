@@ -204,6 +204,9 @@ struct ep_buffer {
     // node of partitions living in this process (ep_buffer_connect): every partition's arena is a peer
     bool connected = false;
     std::vector<ep_buffer*> peers;
+    // how often each phase has been enqueued: the partitions of a node move in lockstep, which lets the
+    // host catch a phase enqueued before the peers' previous phase (nothing on the device waits for it)
+    int64_t num_sends = 0, num_expands = 0, num_partials = 0;
     // state handed from ep_dispatch_launch to ep_dispatch_epilogue_launch
     struct {
         bool valid = false;
@@ -247,6 +250,13 @@ void disconnect(ep_buffer* b) {
     write_peer_table(b, std::vector<char*>(b->num_ranks, b->arena));
     b->connected = false;
     b->peers.clear();
+}
+
+// Phase order inside a node (ep_buffer_connect): `ready(peer)` must hold for every partition.
+template <class F>
+void check_peers(const ep_buffer* b, F&& ready, const char* what) {
+    for (const ep_buffer* p : b->peers)
+        if (not ready(*p)) throw EpError{format("Assertion exception (%s): partition %d of the node: %s", __FILE_NAME__, p->rank_idx, what)};
 }
 
 // The code object is loaded on one device and the arena lives there: calls must come with that
@@ -593,6 +603,12 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             launch(fn, (unsigned)sa.num_row_blocks, EP_ROW_THREADS, 0, a.stream, sa);
         };
 
+        if (num_ranks > 1) {
+            // the rows about to be packed overwrite what the peers received last time
+            check_peers(b, [&](const ep_buffer& p) { return p.num_expands >= b->num_sends; },
+                        "has not run the copy epilogue of the previous dispatch yet");
+            ++b->num_sends;
+        }
         if (cached_mode) {
             // the cached handle already holds the whole layout: only the packed regions are refreshed
             b->last.valid = false;
@@ -680,6 +696,8 @@ int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
         const int R = b->num_ranks;
         if (R == 1) return;             // one partition: ep_dispatch_launch has produced the whole layout
         EP_HOST_ASSERT(b->last.valid and not b->last.recv_done and "follows this buffer's own ep_dispatch_launch");
+        check_peers(b, [&](const ep_buffer& p) { return p.num_sends >= b->num_sends; },
+                    "its ep_dispatch_launch comes before any receive side");
         const int K = a.num_topk, E = a.num_experts;
         EP_HOST_ASSERT(K == b->last.num_topk and E == b->last.num_experts);
         EP_HOST_ASSERT(a.expert_alignment == b->last.alignment and a.num_max_tokens_per_rank == b->last.max_tokens);
@@ -852,6 +870,11 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
             EP_HOST_ASSERT(b->last.num_tokens == num_tokens and b->last.num_topk == K);
             EP_HOST_ASSERT((R == 1 or b->last.recv_done) and "the receive-side layout comes before the copy");
         }
+        if (R > 1) {
+            check_peers(b, [&](const ep_buffer& p) { return p.num_sends >= b->num_sends; },
+                        "its ep_dispatch_launch comes before any copy epilogue");
+            b->num_expands = b->num_sends;
+        }
 
         EpScatterArgs sa{};
         sa.topk_weights = (const float*)a.topk_weights.data;
@@ -1013,6 +1036,10 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
 
         if (phase == 0) {
             if (R == 1) return;     // single partition: the whole reduction is one token-side launch
+            // the partials land where the peers' packed rows are
+            check_peers(b, [&](const ep_buffer& p) { return p.num_expands >= p.num_sends and p.num_sends >= b->num_sends; },
+                        "runs its copy epilogue before any combine");
+            ++b->num_partials;
             // owner side: one partial per received row into this GPU's combine buffer
             ca.y = a.x.data;
             ca.y_row_bytes = (int64_t)hidden * 2;
@@ -1054,6 +1081,8 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             if (grid == 0) return;
             launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, 0, a.stream, ca);
         } else {
+            check_peers(b, [&](const ep_buffer& p) { return p.num_partials >= b->num_partials; },
+                        "its owner-side reduce (phase 0) comes before any token-side reduce");
             // token side: biases + the partial of every master, read from the combine buffer
             ca.y = b->buffer();
             ca.y_row_bytes = combine_token;

@@ -96,7 +96,9 @@ int ep_buffer_create(int rank_idx, int num_ranks, int64_t num_bytes, int64_t num
  * with plain device pointers standing where peer-mapped ones would on several GPUs.  There are no
  * cross-partition waits: the caller orders the launches (every partition's ep_dispatch_launch
  * before any ep_dispatch_recv_launch; every copy epilogue before any combine; every combine phase 0
- * before any phase 1), e.g. by enqueueing them in that order on one stream.  Destroying a
+ * before any phase 1), e.g. by enqueueing them in that order on one stream; the library counts
+ * the phases of every partition and fails a call that comes before its peers' previous phase.
+ * Destroying a
  * partition disconnects the others.  Synchronises.  No counterpart call in the reference, whose
  * ranks find each other through the process group. */
 int ep_buffer_connect(ep_buffer_t** bufs, int n);

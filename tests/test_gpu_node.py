@@ -395,3 +395,31 @@ def test_partitions_connected_by_address():
     for b in bufs:
         b.runtime.set_peers(None)
         b.destroy()
+
+
+def test_node_phase_order_is_checked_on_the_host():
+    """Nothing on the device waits across partitions, so the library refuses a phase whose peers have not
+    enqueued the phase before it: a blocking dispatch inside a node, a combine before every partition has
+    expanded."""
+    import deep_ep
+    R, max_tokens, H, E, K = 2, 16, 64, 4, 2
+    bufs = make_node(R, max_tokens, H, K, False)
+    xs = [make_tokens(max_tokens, H, seed=r).to(DEV) for r in range(R)]
+    routing = [make_routing(max_tokens, E, K, seed=r) for r in range(R)]
+    kw = dict(num_experts=E, num_max_tokens_per_rank=max_tokens, do_expand=True, do_zero_padding=True)
+    # partition 0 wants its receive side before partition 1 has sent anything
+    with pytest.raises(deep_ep._C.EPException, match='partition 1 of the node'):
+        bufs[0].dispatch(xs[0], topk_idx=routing[0][0].to(DEV), topk_weights=routing[0][1].to(DEV), **kw)
+    ev1 = bufs[1].dispatch(xs[1], topk_idx=routing[1][0].to(DEV), topk_weights=routing[1][1].to(DEV),
+                           async_with_compute_stream=True, defer_epilogue=True, **kw)
+    # partition 0's send is enqueued (the failed call got that far); its receive side can run now
+    with pytest.raises(deep_ep._C.EPException, match='previous dispatch'):
+        bufs[0].dispatch(xs[0], topk_idx=routing[0][0].to(DEV), topk_weights=routing[0][1].to(DEV),
+                         async_with_compute_stream=True, defer_epilogue=True, **kw)       # peers have not expanded yet
+    rx1, _, rw1, h1 = ev1.current_stream_wait()
+    # combine of partition 1 before partition 0 has expanded what it received
+    with pytest.raises(deep_ep._C.EPException, match='copy epilogue before any combine'):
+        bufs[1].combine(rx1, h1, topk_weights=rw1, async_with_compute_stream=True, defer_epilogue=True)
+    torch.cuda.synchronize()
+    for b in bufs:
+        b.destroy()
