@@ -485,7 +485,8 @@ __device__ __forceinline__ int64_t region_row_of_stream(const int* psum, int R, 
         q += __popcll(__ballot(before));
     }
     q = min(q, R - 1);
-    return (int64_t)q * max_tokens + (i - (q ? psum[q - 1] : 0));
+    const int slot = min(i - (q ? psum[q - 1] : 0), max_tokens - 1);      // counts of a stale handle cannot lead outside
+    return (int64_t)q * max_tokens + max(slot, 0);
 }
 
 // First byte of the rows that destination j of the task writes, and of their scales.
