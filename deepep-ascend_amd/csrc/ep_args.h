@@ -100,7 +100,7 @@ struct EpScatterArgs {
     int cached;                   // slots come from recv_src_metadata
     int num_sf_packs;             // 2-byte packs per row (prequantised) ; fused: hidden/128 floats
     int num_local_experts, expert_alignment;
-    int zero_padding;
+    int reserved0;
     int num_row_blocks;           // blocks [0, num_row_blocks) copy rows, the rest zero padding
     int num_tokens;               // T: bound of the token indices a row may name
     int num_parts;                // column parts per row; a wave task is (row, part)

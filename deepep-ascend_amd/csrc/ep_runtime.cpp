@@ -900,7 +900,6 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.cached = cached_mode ? 1 : 0;
         sa.num_local_experts = El;
         sa.expert_alignment = a.expert_alignment;
-        sa.zero_padding = a.do_zero_padding ? 1 : 0;
         sa.num_out_rows = (int)std::min<int64_t>(num_expanded, INT32_MAX);
         bool quantise_here = fused;
         if (R == 1) {
