@@ -6,7 +6,7 @@
 #include <stdint.h>
 #include <string.h>
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define EP_HD __host__ __device__ inline
 #else
 #define EP_HD static inline

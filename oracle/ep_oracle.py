@@ -21,6 +21,12 @@ Pinning status of each function (what independent evidence fixes its results):
   reference's own deep_ep/utils/math.py (tests/golden/), by closed forms
   (power-of-two amax, all-zero groups, +-amax -> 0x7E/0xFE) and by an independent
   integer re-implementation of the e4m3fn rounding.
+* no_sync_sizes                         -- pinned by the literal row counts that follow from
+  csrc/buffers/ep.hpp:288,316-320 at the headline shape (130 816 rows with one partition,
+  3 146 752 with 32), a case worked by hand, and a brute-force check that it bounds every
+  layout of random tiny routings.
+* combine_weighted (an extension)       -- pinned by a per-element numpy-float32 loop over slots
+  derived from the closed form, and by reducing to the plain combine when every weight is 1.
 * combine_partial / combine_final       -- pinned by golden vectors produced from the
   reference's own deep_ep/utils/refs.py combine (tests/golden/), by exact cases
   (K=1 identity, powers of two) and by an independent numpy-float32 loop in tests/.

@@ -381,3 +381,88 @@ def test_combine_exact_cases():
     y = torch.full((16, H), 0.25, dtype=torch.bfloat16)
     out, _ = O.combine_fast(y, None, lay['recv_src_metadata'], 4, 4)
     assert torch.all(out == 1.0)
+
+
+# ---------------------------------------------------------------------------------------
+# output sizes without a host sync (csrc/buffers/ep.hpp:288,316-320)
+# ---------------------------------------------------------------------------------------
+def test_no_sync_sizes_literals():
+    # headline shape, one partition: 16384 * min(6, 256) + 127 * 256 = 130 816 rows, a multiple of 128
+    assert O.no_sync_sizes(1, 16384, 6, 256, 128) == (16384, 130816)
+    # 32 partitions of 8 experts: 32 * 16384 * min(6, 8) + 127 * 8 = 3 146 744 -> next multiple of 128
+    assert O.no_sync_sizes(32, 16384, 6, 256, 128) == (524288, 3146752)
+    # by hand: R=2, maxT=4, K=2, E=4 (2 experts a partition), A=2 -> 2*4*min(2,2) + (2-1)*2 = 18
+    assert O.no_sync_sizes(2, 4, 2, 4, 2) == (8, 18)
+    # top-k larger than the local experts: a row has at most one slot per local expert
+    assert O.no_sync_sizes(4, 10, 8, 8, 1) == (40, 4 * 10 * 2)
+    # alignment rounding of the total: 1*3*1 + 4*1 = 7 -> 10
+    assert O.no_sync_sizes(1, 3, 1, 1, 5) == (3, 10)
+
+
+def test_no_sync_sizes_bound_every_layout():
+    # the bound holds for, and is reached by, the layouts it sizes: brute force over tiny routings
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        R = int(rng.integers(1, 4))
+        El = int(rng.integers(1, 4))
+        E, K, A, T = R * El, int(rng.integers(1, 5)), int(rng.integers(1, 6)), int(rng.integers(1, 7))
+        K = min(K, E)
+        topk = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int64)
+        topk[rng.random((T, K)) < 0.2] = -1
+        n_recv_bound, n_exp_bound = O.no_sync_sizes(R, T, K, E, A)
+        assert n_recv_bound == R * T and n_exp_bound % A == 0
+        for r in range(R):
+            lay = O.rank_share_layout(topk, E, R, r, A, T)
+            # a single sender delivers at most T rows and T * min(K, El) slots
+            assert lay['num_recv_tokens'] <= T
+            assert lay['num_expanded_tokens'] <= n_exp_bound
+    # worst case: every partition sends every token to all local experts, counts are 1 mod A
+    R, El, K, A, T = 2, 2, 2, 4, 5
+    cnt = R * T                                  # rows per local expert
+    assert El * O.align(cnt, A) <= O.no_sync_sizes(R, T, K, R * El, A)[1]
+
+
+# ---------------------------------------------------------------------------------------
+# gate-weighted combine (extension): sum_j w_j * y_j in fp32, j ascending, one rounding
+# ---------------------------------------------------------------------------------------
+def test_combine_weighted_brute_force():
+    T, E, K, H, A = 40, 8, 3, 24, 4
+    topk, _ = make_routing(T, E, K, seed=5, masked=0.25)
+    topk[7] = -1
+    lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, T)
+    g = torch.Generator().manual_seed(9)
+    n_exp = lay['num_expanded_tokens']
+    y = torch.randn((n_exp, H), generator=g).to(torch.bfloat16)
+    ew = torch.rand(n_exp, generator=g)
+    got = O.combine_weighted(y, ew, lay['recv_src_metadata'], T, K)
+    # independent per-element loop in numpy float32: the expanded slot of (t, j) from the closed form
+    # slot(t,j) = start[e] + #{earlier (t',j') with the same expert}
+    tk = topk.numpy()
+    cnt = np.zeros(E, np.int64)
+    for t in range(T):
+        for j in range(K):
+            if tk[t, j] >= 0:
+                cnt[tk[t, j]] += 1
+    start = np.zeros(E, np.int64)
+    for e in range(1, E):
+        start[e] = start[e - 1] + (cnt[e - 1] + A - 1) // A * A
+    fill = np.zeros(E, np.int64)
+    yf = y.float().numpy()
+    wf = ew.numpy()
+    exp = np.zeros((T, H), np.float32)
+    for t in range(T):
+        for j in range(K):
+            e = tk[t, j]
+            if e < 0:
+                continue
+            s = start[e] + fill[e]
+            fill[e] += 1
+            for h in range(H):
+                exp[t, h] = np.float32(exp[t, h] + np.float32(wf[s] * yf[s, h]))
+    exp_bf = torch.from_numpy(exp).to(torch.bfloat16)
+    assert torch.equal(got.view(torch.int16), exp_bf.view(torch.int16))
+    # all weights 1 -> the plain combine (more than one slot: same sum, same rounding)
+    ones = torch.ones(n_exp)
+    plain, _ = O.combine_fast(y, None, lay['recv_src_metadata'], T, K)
+    assert torch.equal(O.combine_weighted(y, ones, lay['recv_src_metadata'], T, K).view(torch.int16),
+                       plain.view(torch.int16))
