@@ -141,6 +141,8 @@ int main(void) {
     e.expert_alignment = A;
     e.do_zero_padding = 1;
     e.stream = stream;
+    e.dispatch_stamp = ep_dispatch_stamp(buf);
+    EXPECT(e.dispatch_stamp > 0);
     CHECK_EP(ep_dispatch_epilogue_launch(buf, &e));
 
     /* identity experts: the expanded rows go straight back */

@@ -15,6 +15,7 @@
 #define EP_MAX_PAD_BLOCKS_PER_EXPERT 16
 
 #define EP_LAYOUT_SCANNED 0
+#define EP_LAYOUT_FOLDED 1
 #define EP_LAYOUT_SINGLE 2
 
 #define EP_SCATTER_EXPAND 0

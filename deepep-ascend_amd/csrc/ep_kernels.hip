@@ -23,6 +23,41 @@
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
+// Streaming stores of the row kernels.  The policy bits of the store instruction (sc0, sc1 = scope,
+// nt = non-temporal) decide how the L2 treats the lines; which combination moves rows fastest is a
+// measured choice per kernel (EP_*_ST_POL below; bit 0 = nt, bit 1 = sc0, bit 2 = sc1).
+template <int POL>
+__device__ __forceinline__ void stream_store(u32x4* p, u32x4 v) {
+    if (POL == 0) *p = v;
+    else if (POL == 1) __builtin_nontemporal_store(v, p);
+    else if (POL == 2) asm volatile("global_store_dwordx4 %0, %1, off sc0" ::"v"(p), "v"(v) : "memory");
+    else if (POL == 3) asm volatile("global_store_dwordx4 %0, %1, off sc0 nt" ::"v"(p), "v"(v) : "memory");
+    else if (POL == 4) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    else if (POL == 5) asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" ::"v"(p), "v"(v) : "memory");
+    else if (POL == 6) asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+    else asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" ::"v"(p), "v"(v) : "memory");
+}
+template <int POL>
+__device__ __forceinline__ void stream_store(u32x2* p, u32x2 v) {
+    if (POL == 0) *p = v;
+    else if (POL == 1) __builtin_nontemporal_store(v, p);
+    else if (POL == 2) asm volatile("global_store_dwordx2 %0, %1, off sc0" ::"v"(p), "v"(v) : "memory");
+    else if (POL == 3) asm volatile("global_store_dwordx2 %0, %1, off sc0 nt" ::"v"(p), "v"(v) : "memory");
+    else if (POL == 4) asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    else if (POL == 5) asm volatile("global_store_dwordx2 %0, %1, off sc1 nt" ::"v"(p), "v"(v) : "memory");
+    else if (POL == 6) asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+    else asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1 nt" ::"v"(p), "v"(v) : "memory");
+}
+#ifndef EP_SCATTER_ST_POL
+#define EP_SCATTER_ST_POL 1
+#endif
+#ifndef EP_PAD_ST_POL
+#define EP_PAD_ST_POL 1
+#endif
+#ifndef EP_COMBINE_ST_POL
+#define EP_COMBINE_ST_POL 1
+#endif
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 __device__ __forceinline__ int align_up(int x, int a) { return (x + a - 1) / a * a; }
@@ -228,6 +263,8 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
 //
 // Where the counts of the other blocks come from (a.scan_mode):
 //   EP_LAYOUT_SCANNED  ep_layout_scan left exclusive prefixes in blk_*_cnt and totals in *_total
+//   EP_LAYOUT_FOLDED   ep_layout_count left plain counts in blk_*_cnt: every block sums the rows before it
+//                      itself (cheaper than a launch of its own up to a few hundred blocks)
 //   EP_LAYOUT_SINGLE   one block owns every token: nothing ran before, its own LDS counts are the totals
 // Only the local experts and the partitions need prefixes: slots of other experts are never used.
 // ------------------------------------------------------------------------------------------------
@@ -284,6 +321,25 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
         if (a.scan_mode == EP_LAYOUT_SCANNED) {
             pre[k] = (is_expert ? a.blk_expert_cnt : a.blk_rank_cnt)[(int64_t)b * stride + col];
             tot = is_expert ? a.expert_total[col] : a.rank_total[col];
+        } else if (a.scan_mode == EP_LAYOUT_FOLDED) {
+            // ep_layout_count has finished: this block sums the counts of the blocks before it (and of all
+            // blocks) itself, one column per thread, consecutive threads on consecutive columns of a row
+            const int* base = (is_expert ? a.blk_expert_cnt : a.blk_rank_cnt) + col;
+            const int nb = min(a.num_blocks, max(1, (num_rows + EP_TOKENS_PER_BLOCK - 1) / EP_TOKENS_PER_BLOCK));
+            int before = 0;
+            int r = 0;
+            for (; r + 4 <= nb; r += 4) {
+                const int v0 = base[(int64_t)r * stride], v1 = base[(int64_t)(r + 1) * stride];
+                const int v2 = base[(int64_t)(r + 2) * stride], v3 = base[(int64_t)(r + 3) * stride];
+                before += (r < b ? v0 : 0) + (r + 1 < b ? v1 : 0) + (r + 2 < b ? v2 : 0) + (r + 3 < b ? v3 : 0);
+                tot += v0 + v1 + v2 + v3;
+            }
+            for (; r < nb; ++r) {
+                const int v = base[(int64_t)r * stride];
+                before += r < b ? v : 0;
+                tot += v;
+            }
+            pre[k] = before;
         } else {
             const int* wc = is_expert ? s_we + col : s_wr + col;
             for (int i = 0; i < NW; ++i) tot += wc[i * stride];
@@ -598,7 +654,7 @@ __device__ __forceinline__ void zero_span(char* base, int64_t nbytes, int part, 
     // 16-byte stores over the aligned body; the ends in 2-byte units (every element here is 2 or 4 bytes wide)
     const int64_t head = min((int64_t)((16 - ((uintptr_t)base & 15)) & 15), nbytes);
     const int64_t body = (nbytes - head) & ~(int64_t)15;
-    for (int64_t o = tid * 16; o < body; o += nthreads * 16) __builtin_nontemporal_store(z, (u32x4*)(base + head + o));
+    for (int64_t o = tid * 16; o < body; o += nthreads * 16) stream_store<EP_PAD_ST_POL>((u32x4*)(base + head + o), z);
     for (int64_t o = tid * 2; o < head; o += nthreads * 2) *(unsigned short*)(base + o) = 0;
     for (int64_t o = head + body + tid * 2; o < nbytes; o += nthreads * 2) *(unsigned short*)(base + o) = 0;
 }
@@ -653,7 +709,7 @@ __device__ __forceinline__ void scatter_copy_body(const EpScatterArgs& a) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int v = (part * U + u) * WAVE + lane;
-            if (u < U && v < nvec) __builtin_nontemporal_store(d[u], row + v);
+            if (u < U && v < nvec) stream_store<EP_SCATTER_ST_POL>(row + v, d[u]);
         }
     }
     if (part == 0 && a.recv_sf != nullptr) {
@@ -716,7 +772,7 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
         const int s = readlane(c.myslot, j);
         if (s < 0) continue;
         char* rows = out_rows_of<PACK>(a, c, j);
-        __builtin_nontemporal_store(q8, (u32x2*)(rows + (int64_t)s * a.out_row_bytes) + v);
+        stream_store<EP_SCATTER_ST_POL>((u32x2*)(rows + (int64_t)s * a.out_row_bytes) + v, q8);
         if (writes_scale) ((float*)(out_sf_of<PACK>(a, rows) + (int64_t)s * a.out_sf_row_bytes))[v >> 4] = scale;
     }
 }
@@ -1005,11 +1061,11 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     }
     if (live0) {
         if (MODE == EP_COMBINE_FUSED && has_bias) res0 = add_biases(a, t, v0, true, res0);
-        __builtin_nontemporal_store(res0, out + v0);
+        stream_store<EP_COMBINE_ST_POL>(out + v0, res0);
     }
     if (live1) {
         if (MODE == EP_COMBINE_FUSED && has_bias) res1 = add_biases(a, t, v1, true, res1);
-        __builtin_nontemporal_store(res1, out + v1);
+        stream_store<EP_COMBINE_ST_POL>(out + v1, res1);
     }
 }
 

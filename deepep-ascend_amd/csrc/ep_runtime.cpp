@@ -119,6 +119,7 @@ struct Kernels {
 std::mutex g_mutex;
 Kernels g_k;
 bool g_fp8_hw = true;
+int g_fold_max_blocks = 256;    // up to this many layout workgroups the slot assignment sums the block counts itself
 
 std::string library_dir() {
     Dl_info info;
@@ -199,6 +200,8 @@ struct ep_buffer {
     int* host_page = nullptr;    // pinned + mapped
     int* host_page_dev = nullptr;
     int seq = 0;                 // sequence number of the last non-cached dispatch
+    int64_t launch_stamp = 0;    // counts the non-cached ep_dispatch_launch calls; the latest one owns the workspace
+    int64_t workspace_bytes = kWorkspaceBytes;
     bool destroyed = false;
     int device = 0;
     // node of partitions living in this process (ep_buffer_connect): every partition's arena is a peer
@@ -210,6 +213,7 @@ struct ep_buffer {
     // state handed from ep_dispatch_launch to ep_dispatch_epilogue_launch
     struct {
         bool valid = false;
+        int64_t stamp = 0;
         int num_tokens = 0, num_topk = 0, num_experts = 0, alignment = 0, max_tokens = 0;
         int* slot_map = nullptr;
         int* recv_tok = nullptr;
@@ -225,8 +229,8 @@ struct ep_buffer {
     }
 
     char* workspace() const { return arena; }
-    char* buffer() const { return arena + kWorkspaceBytes; }
-    char* lb() const { return arena + kWorkspaceBytes + num_buffer_bytes; }
+    char* buffer() const { return arena + workspace_bytes; }
+    char* lb() const { return arena + workspace_bytes + num_buffer_bytes; }
 };
 
 namespace {
@@ -240,6 +244,21 @@ unsigned layout_assign_lds(int E, int R, int K) {
     return (unsigned)(E / R + R + nw * (E + R) + nw + 1 + R + nw) * sizeof(int) + layout_key_bytes(K);
 }
 
+// The layout pass: per-block histograms, then the slot assignment.  One block needs no histogram pass; up
+// to g_fold_max_blocks blocks the assignment kernel sums the histograms of the blocks before it itself;
+// beyond that a scan kernel turns them into prefixes first.
+void launch_layout(EpLayoutArgs& la, int num_blocks, void* stream) {
+    const int E = la.num_experts, R = la.num_ranks, K = la.num_topk;
+    const unsigned smem_assign = layout_assign_lds(E, R, K);
+    EP_HOST_ASSERT(smem_assign <= 64 * 1024);
+    la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : (num_blocks <= g_fold_max_blocks ? EP_LAYOUT_FOLDED : EP_LAYOUT_SCANNED);
+    if (la.scan_mode != EP_LAYOUT_SINGLE)
+        launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, layout_count_lds(E, R, K), stream, la);
+    if (la.scan_mode == EP_LAYOUT_SCANNED)
+        launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 16), EP_SCAN_THREADS, 0, stream, la);
+    launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, stream, la);
+}
+
 void write_peer_table(ep_buffer* b, const std::vector<char*>& arenas) {
     std::vector<char*> table(EP_MAX_RANKS, nullptr);
     for (size_t i = 0; i < arenas.size(); ++i) table[i] = arenas[i];
@@ -248,6 +267,8 @@ void write_peer_table(ep_buffer* b, const std::vector<char*>& arenas) {
 
 void disconnect(ep_buffer* b) {
     write_peer_table(b, std::vector<char*>(b->num_ranks, b->arena));
+    // the row counts the other partitions left while connected describe rows nobody will refresh
+    HIP_CHECK(hipMemset(b->arena + EP_WS_INBOX_OFF, 0, sizeof(int) * EP_MAX_RANKS));
     b->connected = false;
     b->peers.clear();
 }
@@ -533,6 +554,10 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         const int packed_sf = a.fused_fp8_quant ? 2 * (int)ceil_div(hidden, 128) : num_sf_packs;
         EP_HOST_ASSERT(dispatch_buffer_size(a.num_max_tokens_per_rank, hidden, packed_sf, num_topk, packed_elem,
                                             num_ranks) <= b->num_buffer_bytes);
+        // packed rows put the scales at the next multiple of 32 bytes behind the payload while the row size adds the
+        // payload unaligned (layout/ep/token.hpp:36-43,59-61, whose own check of this is commented out :29): rows
+        // would overlap their neighbours
+        EP_HOST_ASSERT(num_ranks == 1 or packed_sf == 0 or (int64_t)hidden * packed_elem % kUbAlign == 0);
 
         // handle tensors
         const auto& psum_rank = a.psum_num_recv_tokens_per_rank;
@@ -590,7 +615,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             // unconnected: the regions of this arena, one per destination; in a node: region `rank_idx` of
             // the destination's own arena, where its receive side will look for them
             sa.peer_arenas = b->peer_table();
-            sa.buffer_off = kWorkspaceBytes;
+            sa.buffer_off = b->workspace_bytes;
             sa.region_by_source = b->connected ? 1 : 0;
             sa.num_ranks = num_ranks;
             sa.pack_sf_off = pk.sf_off;
@@ -635,7 +660,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             la.slot_map = carve((int64_t)num_tokens * K);
             la.recv_tok = carve(a.num_max_tokens_per_rank);
         }
-        EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= kWorkspaceBytes);
+        EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= b->workspace_bytes);
         // more than one partition: this launch is the send side only (slots in the destinations' regions, row
         // counts into their inboxes); the receive side is ep_dispatch_recv_launch
         la.send_only = R > 1 ? 1 : 0;
@@ -662,20 +687,12 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         la.cumulative_stats = (int*)a.cumulative_local_expert_recv_stats.data;
         la.host_page = b->host_page_dev;
 
-        const unsigned smem_count = layout_count_lds(E, R, K);
-        const unsigned smem_assign = layout_assign_lds(E, R, K);
-        EP_HOST_ASSERT(smem_assign <= 64 * 1024);
-        // one block: its own counts are the totals and nothing has to run before the slot assignment
-        la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : EP_LAYOUT_SCANNED;
-        if (la.scan_mode != EP_LAYOUT_SINGLE)
-            launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, smem_count, a.stream, la);
-        if (la.scan_mode == EP_LAYOUT_SCANNED)
-            launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 16), EP_SCAN_THREADS, 0, a.stream, la);
-        launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, a.stream, la);
+        launch_layout(la, num_blocks, a.stream);
 
         if (num_ranks > 1) launch_pack();
 
         b->last.valid = true;
+        b->last.stamp = ++b->launch_stamp;
         b->last.num_tokens = num_tokens;
         b->last.num_topk = K;
         b->last.num_experts = E;
@@ -688,6 +705,12 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
     });
 }
 
+int64_t ep_dispatch_stamp(ep_buffer_t* b) {
+    return (b == nullptr || b->destroyed || !b->last.valid) ? 0 : b->last.stamp;
+}
+
+void ep_set_layout_fold_max_blocks(int num_blocks) { g_fold_max_blocks = num_blocks; }
+
 int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
     return guarded([&] {
         EP_HOST_ASSERT(pa != nullptr);
@@ -696,6 +719,7 @@ int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
         const int R = b->num_ranks;
         if (R == 1) return;             // one partition: ep_dispatch_launch has produced the whole layout
         EP_HOST_ASSERT(b->last.valid and not b->last.recv_done and "follows this buffer's own ep_dispatch_launch");
+        EP_HOST_ASSERT(a.dispatch_stamp == b->last.stamp and "the receive side belongs to the latest dispatch launch of this buffer");
         check_peers(b, [&](const ep_buffer& p) { return p.num_sends >= b->num_sends; },
                     "its ep_dispatch_launch comes before any receive side");
         const int K = a.num_topk, E = a.num_experts;
@@ -724,6 +748,7 @@ int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
         EP_HOST_ASSERT(a.hidden_bytes > 0 and a.num_sf_packs >= 0);
         const PackedToken pk = packed_token(a.hidden_bytes, a.num_sf_packs * 2, K, true);
         EP_HOST_ASSERT((int64_t)R * a.num_max_tokens_per_rank * pk.bytes <= b->num_buffer_bytes);
+        EP_HOST_ASSERT(a.num_sf_packs == 0 or a.hidden_bytes % kUbAlign == 0);      // see ep_dispatch_launch
 
         const int num_blocks = std::max<int>(1, (int)ceil_div(rows_bound, EP_TOKENS_PER_BLOCK));
         int* ws = (int*)b->workspace();
@@ -738,7 +763,7 @@ int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
         la.rank_total = carve(R);
         la.blk_expert_cnt = carve((int64_t)num_blocks * E);
         la.blk_rank_cnt = carve((int64_t)num_blocks * R);
-        EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= kWorkspaceBytes and "layout scratch of the receive stream fits the workspace");
+        EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= b->workspace_bytes and "layout scratch of the receive stream fits the workspace");
         la.recv_mode = 1;
         la.num_tokens = (int)rows_bound;
         la.num_topk = K;
@@ -765,14 +790,7 @@ int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
         la.src_off = pk.src_off;
         la.recv_src_metadata = (int*)meta.data;
         la.rows_cap = (int)std::min<int64_t>(meta.size[0], INT32_MAX);
-        la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : EP_LAYOUT_SCANNED;
-        const unsigned smem_assign = layout_assign_lds(E, R, K);
-        EP_HOST_ASSERT(smem_assign <= 64 * 1024);
-        if (la.scan_mode == EP_LAYOUT_SCANNED) {
-            launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, layout_count_lds(E, R, K), a.stream, la);
-            launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 16), EP_SCAN_THREADS, 0, a.stream, la);
-        }
-        launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, a.stream, la);
+        launch_layout(la, num_blocks, a.stream);
         b->last.recv_done = true;
         b->last.notified = a.do_cpu_sync != 0;
     });
@@ -782,6 +800,7 @@ int ep_dispatch_wait_counts(ep_buffer_t* b, int* num_recv_tokens, int* num_expan
     return guarded([&] {
         EP_HOST_ASSERT(b != nullptr and not b->destroyed);
         EP_HOST_ASSERT(b->last.valid);
+        EP_HOST_ASSERT(b->last.notified and "the last dispatch was launched with do_cpu_sync (nothing else publishes the counts)");
         const auto deadline = std::chrono::steady_clock::now() + std::chrono::seconds(b->cpu_timeout_secs);
         volatile int* page = b->host_page;
         while (__atomic_load_n(&page[0], __ATOMIC_ACQUIRE) != b->seq) {
@@ -800,13 +819,14 @@ int ep_dispatch_worst_case_sizes(ep_buffer_t* b, int max_tokens, int num_topk, i
                                  int* num_recv_tokens, int* num_expanded_tokens) {
     return guarded([&] {
         EP_HOST_ASSERT(b != nullptr and not b->destroyed);
-        EP_HOST_ASSERT(num_experts % b->num_ranks == 0 and alignment > 0);
-        const int El = num_experts / b->num_ranks;
-        int64_t n = (int64_t)b->num_ranks * max_tokens * std::min(num_topk, El);
+        const int num_ranks = b->num_ranks;
+        EP_HOST_ASSERT(num_experts % num_ranks == 0 and alignment > 0);
+        const int El = num_experts / num_ranks;
+        int64_t n = (int64_t)num_ranks * max_tokens * std::min(num_topk, El);
         n += (int64_t)(alignment - 1) * El;
         n = align_up(n, alignment);
         EP_HOST_ASSERT(n <= INT32_MAX);
-        *num_recv_tokens = b->num_ranks * max_tokens;
+        *num_recv_tokens = num_ranks * max_tokens;
         *num_expanded_tokens = (int)n;
     });
 }
@@ -867,6 +887,8 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         EP_HOST_ASSERT(present(a.psum_num_recv_tokens_per_expert) and a.psum_num_recv_tokens_per_expert.size[0] == El);
         if (not cached_mode) {
             EP_HOST_ASSERT(b->last.valid and "the copy epilogue follows its own dispatch launch");
+            // the slot map and the receive order live in the workspace, which every dispatch launch overwrites
+            EP_HOST_ASSERT(a.dispatch_stamp == b->last.stamp and "the copy epilogue belongs to the latest dispatch launch of this buffer");
             EP_HOST_ASSERT(b->last.num_tokens == num_tokens and b->last.num_topk == K);
             EP_HOST_ASSERT((R == 1 or b->last.recv_done) and "the receive-side layout comes before the copy");
         }
@@ -920,6 +942,7 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
             const int sf_packs = fused ? 2 * (int)ceil_div(hidden, 128) : num_sf_packs;
             const PackedToken pk = packed_token(hidden * payload_elem, sf_packs * 2, K, not cached_mode);
             EP_HOST_ASSERT((int64_t)R * a.num_max_tokens_per_rank * pk.bytes <= b->num_buffer_bytes);
+            EP_HOST_ASSERT(sf_packs == 0 or (int64_t)hidden * payload_elem % kUbAlign == 0);   // see ep_dispatch_launch
             sa.mode = EP_SCATTER_REGION;
             sa.psum_rank = (const int*)a.psum_num_recv_tokens_per_rank.data;
             sa.num_ranks = R;
@@ -1047,7 +1070,7 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             ca.num_rows_bound = (int)a.src_metadata.size[0];
             ca.combined_x = b->buffer();
             ca.peer_arenas = b->peer_table();
-            ca.buffer_off = kWorkspaceBytes;
+            ca.buffer_off = b->workspace_bytes;
             ca.out_row_bytes = combine_token;
             ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
             if (ca.num_row_blocks == 0) return;

@@ -46,7 +46,8 @@ class _DispatchEpilogueArgs(ctypes.Structure):
         'recv_x', 'recv_sf', 'recv_sf_staging', 'recv_topk_weights', 'recv_src_metadata')] + [
         ('num_topk', ctypes.c_int32), ('num_max_tokens_per_rank', ctypes.c_int32), ('num_experts', ctypes.c_int32),
         ('expert_alignment', ctypes.c_int32), ('cached_mode', ctypes.c_int32), ('do_zero_padding', ctypes.c_int32),
-        ('fused_fp8_quant', ctypes.c_int32), ('recv_sf_layout', ctypes.c_int32), ('stream', ctypes.c_void_p)]
+        ('fused_fp8_quant', ctypes.c_int32), ('recv_sf_layout', ctypes.c_int32), ('stream', ctypes.c_void_p),
+        ('dispatch_stamp', ctypes.c_int64)]
 
 
 class _DispatchRecvArgs(ctypes.Structure):
@@ -56,7 +57,7 @@ class _DispatchRecvArgs(ctypes.Structure):
         ('hidden_bytes', ctypes.c_int32), ('num_sf_packs', ctypes.c_int32), ('num_topk', ctypes.c_int32),
         ('num_max_tokens_per_rank', ctypes.c_int32), ('num_experts', ctypes.c_int32),
         ('expert_alignment', ctypes.c_int32), ('do_cpu_sync', ctypes.c_int32), ('reserved', ctypes.c_int32),
-        ('stream', ctypes.c_void_p)]
+        ('stream', ctypes.c_void_p), ('dispatch_stamp', ctypes.c_int64)]
 
 
 class _CombineArgs(ctypes.Structure):
@@ -102,6 +103,8 @@ _ep_connect = _sig('ep_buffer_connect', ctypes.c_int, ctypes.POINTER(ctypes.c_vo
 _ep_set_peers = _sig('ep_buffer_set_peers', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int)
 _ep_dispatch_epi = _sig('ep_dispatch_epilogue_launch', ctypes.c_int, ctypes.c_void_p,
                         ctypes.POINTER(_DispatchEpilogueArgs))
+_ep_stamp = _sig('ep_dispatch_stamp', ctypes.c_int64, ctypes.c_void_p)
+_ep_set_fold = _sig('ep_set_layout_fold_max_blocks', None, ctypes.c_int)
 _ep_combine = _sig('ep_combine_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_CombineArgs), ctypes.c_int)
 
 
@@ -232,6 +235,12 @@ def fp8_selftest(first: int, count: int, limit: float) -> Tuple[int, int]:
 
 def set_fp8_hw_convert(enable: bool) -> None:
     _ep_set_hw(int(enable))
+
+
+def set_layout_fold_max_blocks(num_blocks: int) -> None:
+    """Tuning: up to this many layout workgroups (128 tokens each) the slot-assignment kernel sums the
+    per-workgroup histograms itself; beyond, a scan kernel runs in between.  Results do not depend on it."""
+    _ep_set_fold(int(num_blocks))
 
 
 class EventHandle:
@@ -419,6 +428,9 @@ class EPBuffer(BufferBase):
         a.cached_mode, a.do_cpu_sync, a.fused_fp8_quant = int(cached_mode), int(do_cpu_sync), int(fused_fp8_quant)
         a.stream = _stream()
         _check(_ep_dispatch(self._h, ctypes.byref(a)))
+        # the epilogue below belongs to this launch: the library refuses it once a later dispatch has
+        # taken over the buffer's workspace
+        stamp = _ep_stamp(self._h)
 
         keep_alive = (x, sf, topk_idx, topk_weights, psum_rank, psum_expert)
 
@@ -447,6 +459,7 @@ class EPBuffer(BufferBase):
                 r.num_topk, r.num_max_tokens_per_rank = num_topk, num_max_tokens_per_rank
                 r.num_experts, r.expert_alignment = num_experts, expert_alignment
                 r.do_cpu_sync = int(do_cpu_sync)
+                r.dispatch_stamp = stamp
                 r.stream = _stream()
                 _check(_ep_dispatch_recv(self._h, ctypes.byref(r)))
 
@@ -519,6 +532,7 @@ class EPBuffer(BufferBase):
             # sizes still unknown on the host: the column stride is the row count the device computed
             e.recv_sf_layout = (2 if num_recv is None else 1) if use_col_major_sf else 0
             e.stream = _stream()
+            e.dispatch_stamp = stamp
             _check(_ep_dispatch_epi(self._h, ctypes.byref(e)))
 
             if num_recv is None:

@@ -202,8 +202,16 @@ class EPBuffer(BufferBase):
             allocate_on_comm_stream: accepted and ignored (there is one stream).
             async_with_compute_stream: also return an event for the enqueued work.
             handle: a previous `EPHandle` to replay (no layout pass, no host sync).
-            do_cpu_sync: read exact counts on the host before allocating outputs (default True
-                without a handle); otherwise outputs have worst-case sizes.
+            do_cpu_sync: read exact counts on the host (default True without a handle); otherwise
+                outputs have worst-case sizes.  With one partition the outputs are allocated for
+                this call's own upper bound (`num_tokens * min(num_topk, num_local_experts) +
+                (expert_alignment - 1) * num_local_experts` rows) so that the copy can be enqueued
+                before the host has the counts, and are returned as views narrowed to the exact
+                sizes: while such a view is alive it keeps the whole bound-sized allocation (up to
+                about 15 % more rows than its shape shows under uniform routing); `.clone()` it to
+                hold only the rows shown.  An epilogue deferred with `defer_epilogue` must run
+                before the next non-cached dispatch is launched on this buffer: the library
+                refuses an epilogue whose dispatch is no longer the buffer's latest.
             do_expand: must be True.  do_handle_copy must be False.
             do_zero_padding: zero the alignment padding rows of the outputs.
             use_tma_aligned_col_major_sf: return the FP8 scales column-major.

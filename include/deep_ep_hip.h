@@ -153,7 +153,18 @@ typedef struct ep_dispatch_recv_args {
     int32_t num_topk, num_max_tokens_per_rank, num_experts, expert_alignment;
     int32_t do_cpu_sync, reserved;
     void* stream;
+    int64_t dispatch_stamp;                             /* ep_dispatch_stamp() taken after this dispatch's ep_dispatch_launch */
 } ep_dispatch_recv_args_t;
+
+/* Stamp of the buffer's latest non-cached ep_dispatch_launch (0: none): hand it to that dispatch's
+ * ep_dispatch_recv_launch / ep_dispatch_epilogue_launch.  No counterpart in the reference, which leaves
+ * the order of deferred epilogues to the caller. */
+int64_t ep_dispatch_stamp(ep_buffer_t* buf);
+
+/* Tuning: number of layout workgroups (128 tokens each) up to which the slot-assignment kernel sums the
+ * per-workgroup histograms itself instead of a scan kernel running in between (default 256).  Results do
+ * not depend on it. */
+void ep_set_layout_fold_max_blocks(int num_blocks);
 
 /* More than one partition, non-cached dispatch: the receive side of launch_dispatch and the slot
  * assignment of the copy epilogue (impls/ep/dispatch.hpp:469-545,
@@ -192,6 +203,11 @@ typedef struct ep_dispatch_epilogue_args {
      * tensor of shape (N_exp,P), strides (1,N_exp) at the start of that storage. */
     int32_t recv_sf_layout;
     void* stream;
+    /* non-cached mode: ep_dispatch_stamp() taken after this dispatch's ep_dispatch_launch.  The slot map the
+     * epilogue reads lives in the buffer's workspace, which the next ep_dispatch_launch overwrites: an epilogue
+     * whose stamp is not the latest fails with an Assertion exception instead of scattering one dispatch's
+     * rows with another's slots (the usage contract of csrc/buffers/ep.hpp:284-286,396-408, enforced). */
+    int64_t dispatch_stamp;
 } ep_dispatch_epilogue_args_t;
 
 /* Expands every received row into its expert-major slots and zeroes the alignment padding:

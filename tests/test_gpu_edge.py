@@ -235,6 +235,53 @@ def test_single_and_multi_block_layouts_agree_with_oracle(T, E, K, R, rank):
     buf.destroy()
 
 
+@pytest.mark.parametrize('T,E,K,R,rank', [(1500, 256, 8, 1, 0), (700, 64, 6, 4, 1)])
+def test_folded_and_scanned_block_prefixes_agree(T, E, K, R, rank):
+    """Several layout workgroups: the slot assignment either sums the histograms of the workgroups before it
+    itself, or reads the prefixes a scan kernel left.  Same handle tensors either way."""
+    import deep_ep
+    H, A = 128, 16
+    topk, w = make_routing(T, E, K, seed=T + 1, masked=0.1)
+    lay = O.rank_share_layout(topk.numpy(), E, R, rank, A, T)
+    try:
+        for fold_max in (256, 1):                        # 1: every multi-block layout takes the scan kernel
+            deep_ep._C.set_layout_fold_max_blocks(fold_max)
+            buf = _buffer(T, H, K, R, rank)
+            _, _, _, handle, _ = buf.dispatch(make_tokens(T, H).to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV),
+                                              num_experts=E, expert_alignment=A, do_expand=True)
+            torch.cuda.synchronize()
+            for name in ('psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
+                         'num_unaligned_recv_tokens_per_expert', 'dst_buffer_slot_idx', 'recv_src_metadata'):
+                assert np.array_equal(getattr(handle, name).cpu().numpy(), lay[name]), (fold_max, name)
+            buf.destroy()
+    finally:
+        deep_ep._C.set_layout_fold_max_blocks(256)
+
+
+def test_epilogue_of_an_overtaken_dispatch_is_refused():
+    """Two deferred dispatches on one buffer: the second launch overwrites the slot map in the buffer's
+    workspace, so the first one's copy epilogue must not run any more; the host refuses it."""
+    import deep_ep
+    T, H, E, K, A = 200, 128, 16, 4, 8
+    buf = _buffer(T, H, K)
+    x = make_tokens(T, H).to(DEV)
+    topk_a, w_a = make_routing(T, E, K, seed=1)
+    topk_b, w_b = make_routing(T, E, K, seed=2)
+    kw = dict(num_experts=E, expert_alignment=A, do_expand=True, do_zero_padding=True,
+              async_with_compute_stream=True, defer_epilogue=True)
+    first = buf.dispatch(x, topk_idx=topk_a.to(DEV), topk_weights=w_a.to(DEV), **kw)
+    second = buf.dispatch(x, topk_idx=topk_b.to(DEV), topk_weights=w_b.to(DEV), **kw)
+    with pytest.raises(deep_ep._C.EPException, match='latest dispatch launch'):
+        first.current_stream_wait()
+    rx, _, rw, handle = second.current_stream_wait()       # the latest one is served, and correctly
+    torch.cuda.synchronize()
+    lay = O.rank_share_layout(topk_b.numpy(), E, 1, 0, A, T)
+    assert np.array_equal(handle.recv_src_metadata.cpu().numpy(), lay['recv_src_metadata'])
+    ex, _, ew = O.rank_share_dispatch(bf16_bits(x.cpu()).view(np.int16), None, w_b.numpy(), lay)
+    assert np.array_equal(bf16_bits(rx).view(np.int16), ex)
+    buf.destroy()
+
+
 def test_plain_c_caller_of_the_abi():
     """deep_ep/lib/abi_client (csrc/abi_client.c, built with gcc): the C ABI used without torch or C++,
     with hipMalloc'd tensors and its own stream; it checks the layout and an exact round trip itself."""

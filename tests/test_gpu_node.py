@@ -72,13 +72,15 @@ NODE_CASES = [
 
 
 # the host sync does not interact with the input format: pre-quantised input runs with it only
-NODE_MODES = [(m, s) for m in ('bf16', 'fp8_fused', 'fp8_prequant') for s in (True, False)
+NODE_MODES = [(m, s) for m in ('bf16', 'fp8_fused', 'fp8_prequant', 'fp8_fused_colmajor') for s in (True, False)
               if s or m != 'fp8_prequant']
 
 
 @pytest.mark.parametrize('R,max_tokens,H,E,K,A,masked', NODE_CASES)
 @pytest.mark.parametrize('mode,do_cpu_sync', NODE_MODES)
 def test_node_dispatch_combine(R, max_tokens, H, E, K, A, masked, mode, do_cpu_sync):
+    col_major = mode.endswith('_colmajor')          # scales asked for as columns; compared as values
+    mode = mode.replace('_colmajor', '')
     bufs = make_node(R, max_tokens, H, K, mode != 'bf16')
     Ts = [max(1, max_tokens - 7 * r) for r in range(R)]                   # ragged token counts
     xs = [make_tokens(T, H, seed=10 * R + r, outliers=True) for r, T in enumerate(Ts)]
@@ -101,7 +103,8 @@ def test_node_dispatch_combine(R, max_tokens, H, E, K, A, masked, mode, do_cpu_s
                                cumulative_local_expert_recv_stats=stats[r], num_experts=E,
                                num_max_tokens_per_rank=max_tokens, expert_alignment=A, do_expand=True,
                                do_zero_padding=True, do_cpu_sync=do_cpu_sync, async_with_compute_stream=True,
-                               defer_epilogue=True, fused_fp8_quant=mode == 'fp8_fused') for r in range(R)]
+                               defer_epilogue=True, fused_fp8_quant=mode == 'fp8_fused',
+                               use_tma_aligned_col_major_sf=col_major) for r in range(R)]
     outs = [ev.current_stream_wait() for ev in events]
     torch.cuda.synchronize()
 
@@ -125,27 +128,43 @@ def test_node_dispatch_combine(R, max_tokens, H, E, K, A, masked, mode, do_cpu_s
         rx, rsf = recv if isinstance(recv, tuple) else (recv, None)
         assert np.array_equal(rx.view(torch.uint8).cpu().numpy().reshape(rx.size(0), -1)[:ne], want[r]['x'])
         if rsf is not None:
+            assert rsf.stride() == ((1, rsf.size(0)) if col_major else (rsf.size(1), 1))
             assert np.array_equal(rsf.contiguous().view(torch.uint8).cpu().numpy().reshape(rsf.size(0), -1)[:ne],
                                   want[r]['sf'])
         assert np.array_equal(rw.cpu().numpy().view(np.uint32)[:ne], want[r]['w'].view(np.uint32))
         handles.append(handle)
 
-    # cached replay through the node: new payload and weights, the layout of the handles
-    if mode == 'bf16' and do_cpu_sync:
-        xs2 = [make_tokens(T, H, seed=30 * R + r) for r, T in enumerate(Ts)]
-        ws2 = [torch.randn(w.shape, generator=torch.Generator().manual_seed(r)).masked_fill(topks[r] < 0, 0)
-               for r, w in enumerate(ws)]
+    # cached replay through the node: new payload and weights, the layout of the handles (packed rows then
+    # carry no routing metadata, which moves the scales and the weights inside them)
+    xs2 = [make_tokens(T, H, seed=30 * R + r) for r, T in enumerate(Ts)]
+    ws2 = [torch.randn(w.shape, generator=torch.Generator().manual_seed(r)).masked_fill(topks[r] < 0, 0)
+           for r, w in enumerate(ws)]
+    quant2 = [O.quantise(x) for x in xs2]
+    if mode == 'bf16':
         rows2 = [bf16_bits(x).view(np.uint8).reshape(x.size(0), -1) for x in xs2]
-        _, want2 = oracle_dispatch(rows2, sfs, [t.numpy() for t in topks], [w.numpy() for w in ws2], E, R, A, max_tokens)
-        evs = [bufs[r].dispatch(xs2[r].to(DEV), topk_weights=ws2[r].to(DEV), handle=handles[r], do_expand=True,
-                                do_zero_padding=True, async_with_compute_stream=True, defer_epilogue=True)
-               for r in range(R)]
-        outs2 = [ev.current_stream_wait() for ev in evs]
-        torch.cuda.synchronize()
-        for r, (rx2, _, rw2, h2) in enumerate(outs2):
-            assert h2 is handles[r]
-            assert np.array_equal(rx2.view(torch.uint8).cpu().numpy().reshape(rx2.size(0), -1), want2[r]['x'])
-            assert np.array_equal(rw2.cpu().numpy().view(np.uint32), want2[r]['w'].view(np.uint32))
+        sfs2 = [None] * R
+        gx2 = [x.to(DEV) for x in xs2]
+    else:
+        rows2 = [q.numpy() for q, _ in quant2]
+        sfs2 = [s_.numpy().view(np.uint8).reshape(s_.size(0), -1) for _, s_ in quant2]
+        gx2 = [x.to(DEV) for x in xs2] if mode == 'fp8_fused' else \
+            [(q.view(torch.float8_e4m3fn).to(DEV), s_.view(torch.int16).to(DEV)) for q, s_ in quant2]
+    _, want2 = oracle_dispatch(rows2, sfs2, [t.numpy() for t in topks], [w.numpy() for w in ws2], E, R, A, max_tokens)
+    evs = [bufs[r].dispatch(gx2[r], topk_weights=ws2[r].to(DEV), handle=handles[r], do_expand=True,
+                            do_zero_padding=True, async_with_compute_stream=True, defer_epilogue=True,
+                            fused_fp8_quant=mode == 'fp8_fused', use_tma_aligned_col_major_sf=col_major)
+           for r in range(R)]
+    outs2 = [ev.current_stream_wait() for ev in evs]
+    torch.cuda.synchronize()
+    for r, (recv2, _, rw2, h2) in enumerate(outs2):
+        assert h2 is handles[r]
+        ne = want[r]['lay']['num_expanded_tokens']
+        rx2, rsf2 = recv2 if isinstance(recv2, tuple) else (recv2, None)
+        assert np.array_equal(rx2.view(torch.uint8).cpu().numpy().reshape(rx2.size(0), -1)[:ne], want2[r]['x'])
+        if rsf2 is not None:
+            assert np.array_equal(rsf2.contiguous().view(torch.uint8).cpu().numpy().reshape(rsf2.size(0), -1)[:ne],
+                                  want2[r]['sf'])
+        assert np.array_equal(rw2.cpu().numpy().view(np.uint32)[:ne], want2[r]['w'].view(np.uint32))
 
     # combine: every owner reduces what it received and sends the partial home
     g = torch.Generator().manual_seed(R)
@@ -423,5 +442,29 @@ def test_node_phase_order_is_checked_on_the_host():
     with pytest.raises(deep_ep._C.EPException, match='copy epilogue before any combine'):
         bufs[1].combine(rx1, h1, topk_weights=rw1, async_with_compute_stream=True, defer_epilogue=True)
     torch.cuda.synchronize()
+    for b in bufs:
+        b.destroy()
+
+
+def test_node_rejects_scaled_rows_that_would_overlap():
+    """Packed rows place the scales at the next multiple of 32 bytes behind the payload while their size adds
+    the payload unaligned (layout/ep/token.hpp:36-43,59-61): with 144 FP8 bytes a row, the metadata of row s
+    would land in row s + 1.  The host refuses instead of corrupting the regions."""
+    import deep_ep
+    R, T, H, E, K = 2, 16, 144, 8, 4
+    bufs = make_node(R, T, H, K, True)
+    topk, w = make_routing(T, E, K)
+    with pytest.raises(deep_ep._C.EPException, match='kUbAlign'):
+        bufs[0].dispatch(make_tokens(T, H).to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV), num_experts=E,
+                         num_max_tokens_per_rank=T, do_expand=True, fused_fp8_quant=True,
+                         async_with_compute_stream=True, defer_epilogue=True)
+    # one partition never materialises packed rows: the same shape is fine there
+    single = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K,
+                              use_fp8_dispatch=True, explicitly_destroy=True)
+    (qx, qs), _, _, _, _ = single.dispatch(make_tokens(T, H).to(DEV), topk_idx=topk.to(DEV), num_experts=E,
+                                           do_expand=True, fused_fp8_quant=True)
+    torch.cuda.synchronize()
+    assert qx.size(1) == H and qs.size(1) == 2
+    single.destroy()
     for b in bufs:
         b.destroy()

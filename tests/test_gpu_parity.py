@@ -368,19 +368,52 @@ def test_contract_violations_raise():
         de._C.calculate_ep_buffer_size(0, 1, 1, 1, False)
 
 
-def test_host_count_wait_times_out():
-    """A dispatch that never notifies the host (do_cpu_sync=False) leaves the count page unarmed; the
-    host wait must give up with the reference's "reduction timeout" after the CPU deadline."""
+def test_host_count_wait_fails_at_once_without_host_sync():
+    """A dispatch launched with do_cpu_sync=False never publishes the counts: waiting for them is a usage
+    error and is reported at once, not after the CPU deadline."""
     import ctypes
+    import time
     de = _deep_ep()
     T, H, E, K = 16, 128, 4, 2
-    buf = _buffer(T, H, K, num_cpu_timeout_secs=1)
+    buf = _buffer(T, H, K, num_cpu_timeout_secs=100)
     topk, _ = make_routing(T, E, K)
     buf.dispatch(make_tokens(T, H).to(DEV), topk_idx=topk.to(DEV), num_experts=E, do_expand=True, do_cpu_sync=False)
     torch.cuda.synchronize()
     a, b = ctypes.c_int(), ctypes.c_int()
+    t0 = time.perf_counter()
     rc = de._C._ep_wait(buf.runtime._h, ctypes.byref(a), ctypes.byref(b), None)
-    assert rc != 0 and 'reduction timeout' in de._C._ep_last_error().decode()
+    assert rc != 0 and 'do_cpu_sync' in de._C._ep_last_error().decode()
+    assert time.perf_counter() - t0 < 5
+    buf.destroy()
+
+
+def test_host_count_wait_times_out():
+    """The counts do not arrive before the CPU deadline: the layout kernels sit behind about two seconds of
+    other work on the stream (a bounded device-side spin that ends by itself), the buffer waits one second.
+    The host gives up with the reference's "reduction timeout"; the stream then drains normally and the
+    buffer is still good."""
+    de = _deep_ep()
+    T, H, E, K = 16, 128, 4, 2
+    buf = _buffer(T, H, K, num_cpu_timeout_secs=1)
+    topk, _ = make_routing(T, E, K)
+    x, tk = make_tokens(T, H).to(DEV), topk.to(DEV)
+    # cycles of the spin kernel per second, measured (its counter need not run at the shader clock)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda._sleep(1000)
+    torch.cuda.synchronize()
+    e0.record()
+    torch.cuda._sleep(20_000_000)
+    e1.record()
+    torch.cuda.synchronize()
+    cycles_per_sec = 20_000_000 / (e0.elapsed_time(e1) * 1e-3)
+    assert 1e6 < cycles_per_sec < 1e11
+    torch.cuda._sleep(int(2.0 * cycles_per_sec))
+    with pytest.raises(de._C.EPException, match='reduction timeout'):
+        buf.dispatch(x, topk_idx=tk, num_experts=E, do_expand=True, do_cpu_sync=True)
+    torch.cuda.synchronize()
+    _, _, _, handle, _ = buf.dispatch(x, topk_idx=tk, num_experts=E, do_expand=True, do_cpu_sync=True)
+    torch.cuda.synchronize()
+    assert handle.num_recv_tokens == T
     buf.destroy()
 
 

@@ -148,6 +148,8 @@ int main(void) {
     printf("%zu %zu\\n", offsetof(ep_combine_args_t, stream), offsetof(ep_combine_args_t, apply_weights));
     printf("%zu %zu %zu\\n", sizeof(ep_dispatch_recv_args_t), offsetof(ep_dispatch_recv_args_t, stream),
            offsetof(ep_dispatch_recv_args_t, hidden_bytes));
+    printf("%zu %zu\\n", offsetof(ep_dispatch_epilogue_args_t, dispatch_stamp),
+           offsetof(ep_dispatch_recv_args_t, dispatch_stamp));
     return 0;
 }
 ''')
@@ -161,7 +163,8 @@ int main(void) {
            C._DispatchEpilogueArgs.stream.offset, C._DispatchEpilogueArgs.recv_sf_layout.offset,
            C._CombineArgs.stream.offset, C._CombineArgs.apply_weights.offset,
            ctypes.sizeof(C._DispatchRecvArgs), C._DispatchRecvArgs.stream.offset,
-           C._DispatchRecvArgs.hidden_bytes.offset]
+           C._DispatchRecvArgs.hidden_bytes.offset,
+           C._DispatchEpilogueArgs.dispatch_stamp.offset, C._DispatchRecvArgs.dispatch_stamp.offset]
     assert got == [int(v) for v in out]
 
 
