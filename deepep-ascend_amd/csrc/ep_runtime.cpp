@@ -19,6 +19,8 @@
 #include "ep_args.h"
 #include "ep_fp8.h"
 
+void ep_static_scratch_init();      // looks up this device's copy of the static scratch (end of this file)
+
 namespace {
 
 constexpr int64_t kAllocAlign = 2097152;       // reference: common/compiled.hpp:48
@@ -202,6 +204,7 @@ struct ep_buffer {
     int seq = 0;                 // sequence number of the last non-cached dispatch
     int64_t launch_stamp = 0;    // counts the non-cached ep_dispatch_launch calls; the latest one owns the workspace
     int64_t workspace_bytes = kWorkspaceBytes;
+    bool is_static = false;      // a view over the library's static scratch: no arena, no count page, one partition
     bool destroyed = false;
     int device = 0;
     // node of partitions living in this process (ep_buffer_connect): every partition's arena is a peer
@@ -296,7 +299,10 @@ extern "C" {
 const char* ep_last_error(void) { return g_err.c_str(); }
 
 int ep_init(const char* dir) {
-    return guarded([&] { load_kernels(dir); });
+    return guarded([&] {
+        load_kernels(dir);
+        ep_static_scratch_init();      // the address of the static scratch on this device
+    });
 }
 
 int64_t ep_get_num_allocation_alignment(void) { return kAllocAlign; }
@@ -492,6 +498,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         const ep_dispatch_args_t& a = *pa;
         const bool cached_mode = a.cached_mode != 0;
         const bool do_cpu_sync = a.do_cpu_sync != 0;
+        EP_HOST_ASSERT(not b->is_static or (not cached_mode and not do_cpu_sync and b->num_ranks == 1));
         if (cached_mode) {
             EP_HOST_ASSERT(not do_cpu_sync and "Cannot do CPU sync with cached mode");
             EP_HOST_ASSERT(not present(a.cumulative_local_expert_recv_stats));
@@ -552,8 +559,9 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         // buffer size (the packed regions of csrc/buffers/ep.hpp:196-198)
         const int packed_elem = a.fused_fp8_quant ? 1 : x_elem;
         const int packed_sf = a.fused_fp8_quant ? 2 * (int)ceil_div(hidden, 128) : num_sf_packs;
-        EP_HOST_ASSERT(dispatch_buffer_size(a.num_max_tokens_per_rank, hidden, packed_sf, num_topk, packed_elem,
-                                            num_ranks) <= b->num_buffer_bytes);
+        // (the static view has no buffer: with one partition the packed regions are never materialised)
+        EP_HOST_ASSERT(b->is_static or dispatch_buffer_size(a.num_max_tokens_per_rank, hidden, packed_sf, num_topk, packed_elem,
+                                                            num_ranks) <= b->num_buffer_bytes);
         // packed rows put the scales at the next multiple of 32 bytes behind the payload while the row size adds the
         // payload unaligned (layout/ep/token.hpp:36-43,59-61, whose own check of this is commented out :29): rows
         // would overlap their neighbours
@@ -660,6 +668,10 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             la.slot_map = carve((int64_t)num_tokens * K);
             la.recv_tok = carve(a.num_max_tokens_per_rank);
         }
+        if (b->is_static and off * (int64_t)sizeof(int) > b->workspace_bytes)
+            throw EpError{format("Assertion exception (%s:%d): the layout scratch of %d tokens x top-%d over %d experts (%lld bytes) "
+                                 "exceeds the library's static scratch of %lld bytes", __FILE_NAME__, __LINE__, num_tokens, K, E,
+                                 (long long)(off * (int64_t)sizeof(int)), (long long)b->workspace_bytes)};
         EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= b->workspace_bytes);
         // more than one partition: this launch is the send side only (slots in the destinations' regions, row
         // counts into their inboxes); the receive side is ep_dispatch_recv_launch
@@ -818,8 +830,8 @@ int ep_dispatch_wait_counts(ep_buffer_t* b, int* num_recv_tokens, int* num_expan
 int ep_dispatch_worst_case_sizes(ep_buffer_t* b, int max_tokens, int num_topk, int num_experts, int alignment,
                                  int* num_recv_tokens, int* num_expanded_tokens) {
     return guarded([&] {
-        EP_HOST_ASSERT(b != nullptr and not b->destroyed);
-        const int num_ranks = b->num_ranks;
+        EP_HOST_ASSERT(b == nullptr or not b->destroyed);
+        const int num_ranks = b == nullptr ? 1 : b->num_ranks;      // no buffer: one partition
         EP_HOST_ASSERT(num_experts % num_ranks == 0 and alignment > 0);
         const int El = num_experts / num_ranks;
         int64_t n = (int64_t)num_ranks * max_tokens * std::min(num_topk, El);
@@ -1119,3 +1131,61 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
 }
 
 }  // extern "C"
+
+// ---- dispatch without any allocation ------------------------------------------------------------
+// For callers that cannot call hipMalloc (code under HIP graph capture, serving loops, harnesses that
+// forbid it): the layout scratch that ep_dispatch_launch carves from a buffer's arena lives in a
+// file-scope device array instead, so no ep_buffer (whose creation allocates) is needed at all.  Every
+// GPU holds its own copy of the array until the process ends; its device address is looked up once per
+// device and kept.  The kernels take that address as an argument, exactly as they take the arena's
+// workspace.  Every call on a GPU shares the array: calls that overlap on one GPU race.  Nothing in it
+// has to start at zero (every word the kernels read was written earlier in the same call).
+#define EP_STATIC_SCRATCH_BYTES (4 * 1024 * 1024)
+static __device__ __align__(256) unsigned char scratch[EP_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+ep_buffer g_static_view[kMaxDevices];       // host-side views: arena = the device's copy of `scratch`
+std::mutex g_static_mutex;
+
+ep_buffer* static_view_of_current_device() {
+    int dev = -1;
+    HIP_CHECK(hipGetDevice(&dev));
+    EP_HOST_ASSERT(dev >= 0 and dev < kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    ep_buffer* v = &g_static_view[dev];
+    if (v->arena == nullptr) {
+        void* ptr = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));     // this device's copy; never the array's name
+        EP_HOST_ASSERT(ptr != nullptr);
+        v->arena = (char*)ptr;
+        v->device = dev;
+        v->rank_idx = 0;
+        v->num_ranks = 1;
+        v->num_buffer_bytes = 0;
+        v->workspace_bytes = EP_STATIC_SCRATCH_BYTES;
+        v->is_static = true;
+    }
+    return v;
+}
+}  // namespace
+
+void ep_static_scratch_init() { (void)static_view_of_current_device(); }
+
+extern "C" int ep_dispatch_static_launch(const ep_dispatch_args_t* d, const ep_dispatch_epilogue_args_t* e) {
+    int rc = guarded([&] {
+        EP_HOST_ASSERT(d != nullptr and e != nullptr);
+        load_kernels(nullptr);
+        EP_HOST_ASSERT(not d->cached_mode and not d->do_cpu_sync and not e->cached_mode);
+        EP_HOST_ASSERT(d->stream == e->stream);
+    });
+    if (rc != 0) return rc;
+    ep_buffer* v = nullptr;
+    rc = guarded([&] { v = static_view_of_current_device(); });
+    if (rc != 0) return rc;
+    rc = ep_dispatch_launch(v, d);
+    if (rc != 0) return rc;
+    ep_dispatch_epilogue_args_t ee = *e;
+    ee.dispatch_stamp = v->last.stamp;
+    return ep_dispatch_epilogue_launch(v, &ee);
+}

@@ -105,6 +105,8 @@ _ep_dispatch_epi = _sig('ep_dispatch_epilogue_launch', ctypes.c_int, ctypes.c_vo
                         ctypes.POINTER(_DispatchEpilogueArgs))
 _ep_stamp = _sig('ep_dispatch_stamp', ctypes.c_int64, ctypes.c_void_p)
 _ep_set_fold = _sig('ep_set_layout_fold_max_blocks', None, ctypes.c_int)
+_ep_dispatch_static = _sig('ep_dispatch_static_launch', ctypes.c_int, ctypes.POINTER(_DispatchArgs),
+                           ctypes.POINTER(_DispatchEpilogueArgs))
 _ep_combine = _sig('ep_combine_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_CombineArgs), ctypes.c_int)
 
 

@@ -21,7 +21,9 @@ DEVICE_FLAGS = [
     '-fhip-fp32-correctly-rounded-divide-sqrt',       # 448/amax and amax/448 are IEEE divisions
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
 ]
-HOST_FLAGS = ['-shared', '-fPIC', '-O2', '-std=c++17', '-Wall']
+# the runtime is compiled as HIP: it holds one device array (the static scratch of ep_dispatch_static_launch)
+HOST_FLAGS = ['-x', 'hip', '--offload-arch=gfx950', '-shared', '-fPIC', '-O2', '-std=c++17', '-Wall',
+              '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']
 ROCM = os.environ.get('ROCM_PATH', '/opt/rocm')
 C_CLIENT_FLAGS = ['-std=c11', '-O1', '-Wall', '-D__HIP_PLATFORM_AMD__', f'-I{ROCM}/include']
 

@@ -181,7 +181,7 @@ int ep_dispatch_recv_launch(ep_buffer_t* buf, const ep_dispatch_recv_args_t* arg
  * timeout ("reduction timeout").  per_expert receives E/R aligned counts.  Replaces the
  * reduction::host::wait_ready loop of csrc/buffers/ep.hpp:295-315. */
 int ep_dispatch_wait_counts(ep_buffer_t* buf, int* num_recv_tokens, int* num_expanded_tokens, int* per_expert);
-/* Worst-case sizes without a host sync (csrc/buffers/ep.hpp:288,316-320). */
+/* Worst-case sizes without a host sync (csrc/buffers/ep.hpp:288,316-320).  buf == NULL: one partition. */
 int ep_dispatch_worst_case_sizes(ep_buffer_t* buf, int num_max_tokens_per_rank, int num_topk, int num_experts,
                                  int expert_alignment, int* num_recv_tokens, int* num_expanded_tokens);
 
@@ -213,6 +213,18 @@ typedef struct ep_dispatch_epilogue_args {
 /* Expands every received row into its expert-major slots and zeroes the alignment padding:
  * replaces launch_dispatch_copy_epilogue (csrc/kernels/ep/dispatch.hpp:84-139). */
 int ep_dispatch_epilogue_launch(ep_buffer_t* buf, const ep_dispatch_epilogue_args_t* args);
+
+/* A whole single-partition dispatch without a host sync (ep_dispatch_launch followed by
+ * ep_dispatch_epilogue_launch, non-cached, do_cpu_sync = 0) that needs no ep_buffer and allocates
+ * nothing: the layout scratch lives in a 4 MiB device array inside the library instead of a buffer's
+ * arena.  It has no counterpart in the reference; it is for callers that cannot allocate (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The caller passes every
+ * input and output, the outputs sized by ep_dispatch_worst_case_sizes(NULL, ...);
+ * epilogue_args->dispatch_stamp is ignored.  Fails with a clear message when the scratch the shape needs (about
+ * 4 * (T*K + max_tokens + ceil(T/128) * (E + 64)) bytes) exceeds the array.  Results equal those of the
+ * two calls it stands for.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (different streams, or host threads) race; calls on one stream are ordered and safe. */
+int ep_dispatch_static_launch(const ep_dispatch_args_t* args, const ep_dispatch_epilogue_args_t* epilogue_args);
 
 /* ---- combine --------------------------------------------------------------------------------- */
 
