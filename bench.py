@@ -25,11 +25,41 @@ import numpy as np  # noqa: E402
 import torch  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch on the headline workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
-# what the same counter reads for a plain 1 GiB copy (x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE):
-# profiles/headline_dispatch_combine_hbm_traffic.txt.  The scatter figure includes the zero padding.
-MEASURED_TRAFFIC = {('c3_headline', 'ep_scatter_quant'): 241.1e6 + 844.9e6,
-                    ('c3_headline', 'ep_combine_k6'): 1417.1e6 + 235.7e6}
+# HBM bytes per launch come from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of a workload
+# (lines "traffic_bytes <kernel> <bytes>"), and only while that summary was taken from the kernel sources
+# that are being run (line "kernel_source_sha256 <hash>"); otherwise the field is null.
+TRAFFIC_PROFILES = {'c3_headline': 'headline_dispatch_combine_hbm_traffic.txt'}
+KERNEL_SOURCES = ('deepep-ascend_amd/csrc/ep_kernels.hip', 'deepep-ascend_amd/csrc/ep_args.h',
+                  'deepep-ascend_amd/csrc/ep_fp8.h')
+
+
+def kernel_source_sha256():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), 'rb') as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic(workload):
+    """{kernel: HBM bytes per launch} from the committed counter summary of this workload, or {} when there
+    is none or it was taken from other kernel sources."""
+    name = TRAFFIC_PROFILES.get(workload)
+    path = os.path.join(ROOT, 'profiles', name) if name else None
+    if not path or not os.path.exists(path):
+        return {}, 'no counter summary committed for this workload'
+    sha, out = None, {}
+    with open(path) as f:
+        for line in f:
+            w = line.split()
+            if len(w) == 2 and w[0] == 'kernel_source_sha256':
+                sha = w[1]
+            elif len(w) == 3 and w[0] == 'traffic_bytes':
+                out[w[1]] = float(w[2])
+    if sha != kernel_source_sha256():
+        return {}, f'profiles/{name} was taken from other kernel sources'
+    return out, f'profiles/{name}'
 WORKLOADS = {
     # name: (T, H, E, K, A, fp8)
     'c3_headline': (16384, 7168, 256, 6, 128, True),
@@ -65,9 +95,29 @@ def make_inputs(T, H, E, K, seed=0):
     return x, topk, w
 
 
+def cpu_small_case():
+    """The reference's CPU-runnable case (128 tokens x 256, 8 experts, top-2, alignment 1, BF16 dispatch then
+    combine of the dispatched rows) on the host cores: median of 5 passes of the oracle."""
+    from oracle import ep_oracle as O
+    T, H, E, K, A, _ = WORKLOADS['c1_small']
+    x, topk, w = make_inputs(T, H, E, K, seed=1)
+    ts = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, T)
+        rx, _, rw = O.rank_share_dispatch(x.view(torch.int16).numpy(), None, w.numpy(), lay)
+        O.combine_fast(torch.from_numpy(rx).view(torch.bfloat16), torch.from_numpy(rw), lay['recv_src_metadata'], T, K)
+        ts.append(time.perf_counter() - t0)
+    n_valid = int(lay['num_unaligned_recv_tokens_per_expert'].sum())
+    nbytes = dispatch_bytes(T, H, K, n_valid, lay['num_recv_tokens'], False, False) + \
+        combine_bytes(T, H, K, n_valid, lay['num_recv_tokens'], 0, True)
+    med = sorted(ts)[len(ts) // 2]
+    return {'workload': 'c1_small', 'ms': round(med * 1e3, 3), 'gbs': round(nbytes / med / 1e9, 3)}
+
+
 def cpu_baseline(H, E, K, A, fp8, sample_tokens, budget_s=12.0, max_passes=16):
     """The oracle on the host cores: whole passes over `sample_tokens` tokens of the same workload, repeated
-    until about `budget_s` seconds of CPU work have been spent."""
+    until about `budget_s` seconds of CPU work have been spent; and the reference's own CPU-runnable case."""
     from oracle import ep_oracle as O
     torch.set_num_threads(os.cpu_count())
     x, topk, w = make_inputs(sample_tokens, H, E, K, seed=1)
@@ -99,7 +149,37 @@ def cpu_baseline(H, E, K, A, fp8, sample_tokens, budget_s=12.0, max_passes=16):
     secs = t_dispatch + t_combine
     return {'value': round(nbytes / secs / 1e9, 3), 'unit': 'GB/s', 'cores': torch.get_num_threads(), 'kind': 'port',
             'sample': f'{passes} passes over {sample_tokens} tokens of the workload: dispatch {t_dispatch:.2f} s + '
-                      f'combine {t_combine:.2f} s of numpy/torch-CPU oracle (os.cpu_count()={os.cpu_count()})'}
+                      f'combine {t_combine:.2f} s of numpy/torch-CPU oracle (os.cpu_count()={os.cpu_count()})',
+            'small_case': cpu_small_case()}
+
+
+def calibrate_write(deep_ep, timed, n, dispatch, handle, T, H, K, n_valid, n_recv, pad_bytes, dev, us_scatter):
+    """Pure writes of the byte count the fused FP8 copy kernel writes (payload, scales, weights, metadata, zero
+    padding), same sampling as the kernels: 4 KiB chunks in address order, in scrambled order, torch's fill,
+    and the copy kernel itself with its loads of x taken out (same stores to the same slots)."""
+    wbytes = n_valid * (H + (H // 128) * 4 + 4) + n_recv * (K + 2) * 4 + pad_bytes
+    seq_bytes = -(-wbytes // 4096) * 4096
+    pow2_bytes = 4096 << (seq_bytes // 4096 - 1).bit_length()          # the scrambled order needs 2^k chunks
+    area = torch.empty(pow2_bytes, dtype=torch.uint8, device=dev)
+    med = lambda v: v[len(v) // 2]  # noqa: E731
+    res = {'copy_kernel_write_bytes': wbytes}
+
+    def entry(name, us, nbytes, note):
+        res[name] = {'us': round(us, 2), 'bytes': nbytes, 'gbs': round(nbytes / us / 1e3, 1), 'what': note}
+
+    entry('ep_calib_fill', med(timed(lambda: deep_ep._C.calibrate_fill(area[:seq_bytes]), n)), seq_bytes,
+          '4 KiB per workgroup, one 16-byte non-temporal store per thread, address order')
+    entry('ep_calib_fill_shuffled', med(timed(lambda: deep_ep._C.calibrate_fill(area, shuffled=True), n)), pow2_bytes,
+          'the same chunks in a scrambled order')
+    entry('torch_fill', med(timed(lambda: area[:seq_bytes].zero_(), n)), seq_bytes, 'torch zero_() of the same bytes')
+    deep_ep._C.set_calibration_stores_only(True)
+    try:
+        us = med(timed(lambda: dispatch(handle), n))
+    finally:
+        deep_ep._C.set_calibration_stores_only(False)
+    entry('ep_scatter_quant_stores_only', us, wbytes, 'the copy kernel without its loads of x: same tasks, same stores')
+    res['ep_scatter_quant'] = {'us': round(us_scatter, 2), 'what': 'the copy kernel (reads x, writes the same bytes)'}
+    return res
 
 
 def timed_us(fn, n):
@@ -281,6 +361,11 @@ def main():
                     help='per-kernel samples back to back, without rewriting a 1 GiB scratch buffer between them')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run a plain 1 GiB device copy (known traffic) to scale rocprof byte counters')
+    ap.add_argument('--calibrate-write', action='store_true',
+                    help='also time pure writes of the copy kernel\'s byte count: 4 KiB chunks in address order '
+                         '(ep_calib_fill), in scrambled order (ep_calib_fill_shuffled), torch\'s fill, and the copy '
+                         'kernel with its loads taken out (ep_scatter_quant_stores_only)')
+    ap.add_argument('--samples', type=int, default=50, help='isolated, cache-flushed launches per kernel')
     args = ap.parse_args()
     if args.graph:
         args.no_cpu_sync = True     # a graph cannot hold the host's wait for the counts
@@ -367,14 +452,16 @@ def main():
         loop_dispatch = sorted(m[0].elapsed_time(m[1]) * 1e3 for m in marks)
         loop_combine = sorted(m[1].elapsed_time(m[2]) * 1e3 for m in marks)
 
-    # Isolated samples, a few: the copy kernel alone is what a cached dispatch enqueues.
-    # Between samples a 1 GiB scratch buffer is rewritten, so no sample finds its inputs in the L2 or
-    # the memory-side cache (the reference's benchmark does the same: tests/ep/test_ep.py:79-80,415-421).
+    # Isolated samples: the copy kernel alone is what a cached dispatch enqueues.  Ten untimed launches, then
+    # --samples timed ones; before each a 1 GiB scratch buffer is rewritten, so no sample finds its inputs in
+    # the L2 or the memory-side cache (the reference's benchmark does the same: tests/ep/test_ep.py:79-80,
+    # 415-421).  The median is reported (the mean beside it).
     scratch = None if args.no_flush else torch.empty(1 << 30, dtype=torch.uint8, device=dev)
 
-    def timed(fn, n):
+    def timed(fn, n, warm=10):
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
-        fn()                                                          # one untimed call first
+        for _ in range(warm):
+            fn()
         for a, b in evs:
             if scratch is not None:
                 scratch.zero_()
@@ -384,21 +471,22 @@ def main():
         torch.cuda.synchronize()
         return sorted(a.elapsed_time(b) * 1e3 for a, b in evs)      # microseconds
 
-    n_k = 10
+    n_k = args.samples
     t_scatter = timed(lambda: dispatch(handle), n_k)
     t_combine = timed(lambda: buf.combine(y, handle, topk_weights=recv_w), n_k)
     t_dispatch_full = timed(lambda: dispatch(), n_k)
     avg = lambda v: sum(v) / len(v)  # noqa: E731
     med = lambda v: v[len(v) // 2]  # noqa: E731
-    us_scatter, us_combine, us_dispatch = med(t_scatter), med(t_combine), med(t_dispatch_full)
+    us_scatter = med(t_scatter)
+    traffic, traffic_source = measured_traffic(args.workload) if not args.no_cpu_sync else ({}, 'not the profiled configuration')
 
     def roof(name, nbytes, samples):
-        us = avg(samples)
+        us = med(samples)
         gbs = nbytes / us / 1e3
-        traffic = MEASURED_TRAFFIC.get((args.workload, name)) if not args.no_cpu_sync else None
         return {'kernel': name, 'bound': 'hbm', 'achieved': round(gbs, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': round(gbs / HBM_PEAK_GBS, 4), 'traffic': traffic, 'us': round(us, 2),
-                'us_median': round(med(samples), 2), 'bytes': nbytes}
+                'frac': round(gbs / HBM_PEAK_GBS, 4), 'traffic': traffic.get(name), 'us': round(us, 2),
+                'us_mean': round(avg(samples), 2), 'us_min': round(samples[0], 2), 'samples': len(samples),
+                'bytes': nbytes}
 
     scatter_name = 'ep_scatter_quant' if fp8 else 'ep_scatter_copy'
     kernels = [roof(scatter_name, b_d, t_scatter), roof(f'ep_combine_k{K}', b_c, t_combine)]
@@ -408,9 +496,21 @@ def main():
     # stream: the kernel plus the gap to its predecessor).
     if loop_combine is not None:
         dominant = roof(f'ep_combine_k{K}', b_c, loop_combine)
-        us_dispatch, us_combine = avg(loop_dispatch), avg(loop_combine)
+        us_dispatch, us_combine = med(loop_dispatch), med(loop_combine)
     else:
         dominant = max(kernels, key=lambda k: k['us'])
+        us_dispatch, us_combine = med(t_dispatch_full), med(t_combine)
+    roofline = {k: dominant[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'traffic')}
+    roofline.update({
+        'kernel': dominant['kernel'], 'traffic_source': traffic_source,
+        # both kernels of the path, each alone (median of the isolated, flushed launches), as fractions of 8 TB/s
+        'dispatch_kernel': scatter_name, 'dispatch_frac': kernels[0]['frac'], 'dispatch_achieved': kernels[0]['achieved'],
+        'dispatch_traffic': kernels[0]['traffic'],
+        'dispatch_frac_incl_zero_padding': round((b_d + pad_bytes) / us_scatter / 1e3 / HBM_PEAK_GBS, 4),
+        'combine_kernel': kernels[1]['kernel'], 'combine_frac': kernels[1]['frac'], 'combine_achieved': kernels[1]['achieved'],
+        'combine_traffic': kernels[1]['traffic'],
+        # the dispatch phase inside the timed region: layout kernels + copy kernel (+ the gaps between them)
+        'dispatch_phase_frac': round(b_d / us_dispatch / 1e3 / HBM_PEAK_GBS, 4)})
     out = {
         'metric': 'dispatch & combine GB/s + % of HBM peak, 16384 tok x7168, top-6/256, FP8/BF16',
         'value': round((b_d + b_c) / ms_per_step / 1e6, 1), 'unit': 'GB/s',
@@ -424,12 +524,12 @@ def main():
                    'do_zero_padding': True, 'do_cpu_sync': not args.no_cpu_sync, 'hip_graph': bool(args.graph),
                    'cache_flush_between_kernel_samples': not args.no_flush,
                    'num_valid_rows': n_valid, 'num_expanded_rows': n_exp_exact},
-        'roofline': {k: dominant[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'traffic')} |
-                    {'kernel': dominant['kernel']},
+        'roofline': roofline,
         'kernels': kernels,
         'phases': {
-            'measured': 'inside the timed region' if loop_combine is not None else 'isolated launches',
+            'measured': 'inside the timed region, medians' if loop_combine is not None else 'isolated launches, medians',
             'dispatch_us': round(us_dispatch, 2), 'dispatch_layout_and_host_sync_us': round(us_dispatch - us_scatter, 2),
+            'dispatch_isolated_flushed_us': round(med(t_dispatch_full), 2),
             'dispatch_gbs': round(b_d / us_dispatch / 1e3, 1), 'dispatch_frac_hbm': round(b_d / us_dispatch / 1e3 / HBM_PEAK_GBS, 4),
             'combine_us': round(us_combine, 2), 'combine_gbs': round(b_c / us_combine / 1e3, 1),
             'combine_frac_hbm': round(b_c / us_combine / 1e3 / HBM_PEAK_GBS, 4),
@@ -437,6 +537,9 @@ def main():
             'scatter_gbs_incl_padding': round((b_d + pad_bytes) / us_scatter / 1e3, 1),
         },
     }
+    if args.calibrate_write and fp8:
+        out['write_calibration'] = calibrate_write(deep_ep, timed, n_k, dispatch, handle, T, H, K, n_valid, n_recv,
+                                                   pad_bytes, dev, us_scatter)
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(H, E, K, A, fp8, min(args.cpu_sample_tokens, T))
     buf.destroy()

@@ -51,10 +51,11 @@ struct EpLayoutArgs {
     int notify_host;              // do_cpu_sync
     int scan_mode;                // EP_LAYOUT_*: where ep_layout_assign finds the other blocks' counts
     // scratch (device)
-    int* blk_expert_cnt;          // [num_blocks, E]   counts, then exclusive prefix over blocks
-    int* blk_rank_cnt;            // [num_blocks, R]   master counts, then exclusive prefix
-    int* expert_total;            // [E]
-    int* rank_total;              // [R]
+    int* blk_cnt;                 // [num_blocks, cnt_stride]  per workgroup: entries per local expert (columns [0, El)),
+                                  //   masters per partition (columns [El, El + R)), zeros up to the stride; after
+                                  //   ep_layout_scan the exclusive prefix over the workgroups instead
+    int* col_total;               // [cnt_stride]  column totals (written by ep_layout_scan)
+    int cnt_stride;               // El + R rounded up to a multiple of 4 ints
     int* slot_map;                // [T, K]  expanded slot of (t, j) if its expert is local, else -1
     int* recv_tok;                // [max_tokens]  receive-stream row -> local token index
     // handle tensors (device)
@@ -178,4 +179,11 @@ struct EpFp8TestArgs {
     unsigned long long* out;      // [0] mismatches, [1] first mismatching pattern
     float limit;                  // only |x| <= limit is compared (NaN patterns are skipped)
     int pad;
+};
+
+// Calibration fill: num_chunks chunks of 4 KiB starting at dst.
+struct EpCalibArgs {
+    void* dst;
+    unsigned num_chunks;
+    unsigned value;
 };

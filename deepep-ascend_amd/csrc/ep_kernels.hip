@@ -120,12 +120,16 @@ __device__ __forceinline__ int64_t recv_packed_row(const int* psum, int R, int m
 
 // Stages the expert ids of this workgroup's entries.  Send side: entry (t, j) of topk_idx.  Receive
 // side: entry (row, j) of the receive stream, read from the packed row; partitions play no role there.
-// Returns the number of rows (tokens) the entries range over.
-__device__ __forceinline__ int layout_load_keys(const EpLayoutArgs& a, short* s_key, short* s_rk, int* s_psum) {
+// num_rows: rows (tokens) the entries range over (layout_num_rows).
+__device__ __forceinline__ int layout_num_rows(const EpLayoutArgs& a, int* s_psum) {
+    return a.recv_mode ? recv_scan_sources(a, s_psum) : a.num_tokens;
+}
+__device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s_key, short* s_rk, const int* s_psum,
+                                                 int num_rows) {
     const int K = a.num_topk;
     const int n = EP_TOKENS_PER_BLOCK * K;
     if (a.recv_mode) {
-        const int N = recv_scan_sources(a, s_psum);
+        const int N = num_rows;
         for (int i = threadIdx.x; i < n; i += blockDim.x) {
             const int row = i / K, j = i - row * K;
             const int g = blockIdx.x * EP_TOKENS_PER_BLOCK + row;
@@ -138,7 +142,7 @@ __device__ __forceinline__ int layout_load_keys(const EpLayoutArgs& a, short* s_
             s_key[i] = (short)e;
             s_rk[i] = -1;
         }
-        return N;
+        return;
     }
     const int64_t base = (int64_t)blockIdx.x * n;
     const int64_t total = (int64_t)a.num_tokens * K;
@@ -151,7 +155,6 @@ __device__ __forceinline__ int layout_load_keys(const EpLayoutArgs& a, short* s_
         s_key[i] = (short)e;
         s_rk[i] = (short)(e < 0 ? -1 : e / a.experts_per_rank);
     }
-    return a.num_tokens;
 }
 
 // Destination partition of entry idx if it is the last slot of its token going there, else -1
@@ -178,9 +181,10 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(
     short* s_rk = s_key + EP_TOKENS_PER_BLOCK * K;
     int* s_psum = (int*)(s_rk + EP_TOKENS_PER_BLOCK * K);      // [R + waves]  (receive side)
     for (int i = threadIdx.x; i < E + R; i += blockDim.x) smem[i] = 0;
-    const int num_rows = layout_load_keys(a, s_key, s_rk, s_psum);
+    const int num_rows = layout_num_rows(a, s_psum);
     // the scan stops at the last workgroup that has rows: the ones behind it leave nothing
     if ((int)blockIdx.x > 0 && (int)blockIdx.x * EP_TOKENS_PER_BLOCK >= num_rows) return;
+    layout_load_keys(a, s_key, s_rk, s_psum, num_rows);
     __syncthreads();
     const int n = EP_TOKENS_PER_BLOCK * K;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -190,8 +194,11 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(
         if (mr >= 0) atomicAdd(&s_rcnt[mr], 1);
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < E; i += blockDim.x) a.blk_expert_cnt[(int64_t)blockIdx.x * E + i] = s_ecnt[i];
-    for (int i = threadIdx.x; i < R; i += blockDim.x) a.blk_rank_cnt[(int64_t)blockIdx.x * R + i] = s_rcnt[i];
+    // one row of the count matrix: this partition's experts, then the partitions, then zero fill
+    const int El = a.experts_per_rank, lo = a.rank_idx * El;
+    int* row = a.blk_cnt + (int64_t)blockIdx.x * a.cnt_stride;
+    for (int i = threadIdx.x; i < a.cnt_stride; i += blockDim.x)
+        row[i] = i < El ? s_ecnt[lo + i] : (i < El + R ? s_rcnt[i - El] : 0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -205,7 +212,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(
 extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpLayoutArgs a) {
     __shared__ int s_part[EP_SCAN_GROUPS][EP_SCAN_COLS + 1];
     __shared__ int s_rows;
-    const int E = a.num_experts, R = a.num_ranks;
+    const int R = a.num_ranks, W = a.cnt_stride;
     int B = a.num_blocks;
     if (a.recv_mode) {
         // rows exist only up to the length of the receive stream
@@ -217,18 +224,13 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
     }
     const int c = threadIdx.x % EP_SCAN_COLS, g = threadIdx.x / EP_SCAN_COLS;
     const int col = blockIdx.x * EP_SCAN_COLS + c;
-    const bool live = col < E + R;
-    int* base = nullptr;
-    int stride = 0;
-    if (live) {
-        if (col < E) { base = a.blk_expert_cnt + col; stride = E; }
-        else { base = a.blk_rank_cnt + (col - E); stride = R; }
-    }
+    const bool live = col < W;
+    int* base = a.blk_cnt + col;
     const int rpg = (B + EP_SCAN_GROUPS - 1) / EP_SCAN_GROUPS;
     const int r0 = min(B, g * rpg), r1 = min(B, r0 + rpg);
     int sum = 0;
     if (live)
-        for (int r = r0; r < r1; ++r) sum += base[(int64_t)r * stride];
+        for (int r = r0; r < r1; ++r) sum += base[(int64_t)r * W];
     s_part[g][c] = sum;
     __syncthreads();
     int off = 0, total = 0;
@@ -240,14 +242,11 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
     if (live) {
         int run = off;
         for (int r = r0; r < r1; ++r) {
-            const int v = base[(int64_t)r * stride];
-            base[(int64_t)r * stride] = run;
+            const int v = base[(int64_t)r * W];
+            base[(int64_t)r * W] = run;
             run += v;
         }
-        if (g == 0) {
-            if (col < E) a.expert_total[col] = total;
-            else a.rank_total[col - E] = total;
-        }
+        if (g == 0) a.col_total[col] = total;
     }
 }
 
@@ -268,6 +267,8 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
 //   EP_LAYOUT_SINGLE   one block owns every token: nothing ran before, its own LDS counts are the totals
 // Only the local experts and the partitions need prefixes: slots of other experts are never used.
 // ------------------------------------------------------------------------------------------------
+#define EP_FOLD_DEPTH 22
+#define EP_KEY_MASTER 0x4000          // flag in a staged key: the entry is the master of its partition (ids < 2048)
 #define EP_LAYOUT_MAX_COLS_PER_THREAD ((EP_MAX_EXPERTS + EP_MAX_RANKS + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS)
 
 extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign(EpLayoutArgs a) {
@@ -286,10 +287,75 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     const int lo = a.rank_idx * El;
     const int ncols = El + R;              // column c < El: local expert lo + c; else partition c - El
 
+    const int num_rows = layout_num_rows(a, s_psum);
+    if (b > 0 && b * EP_TOKENS_PER_BLOCK >= num_rows) return;      // nothing to rank here, nothing to publish
+
+    // ---- counts of the workgroups before this one (kept in registers) and totals over all of them ----
+    int pre[EP_LAYOUT_MAX_COLS_PER_THREAD], tot[EP_LAYOUT_MAX_COLS_PER_THREAD];
+#pragma unroll
+    for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) pre[k] = tot[k] = 0;
+    if (a.scan_mode == EP_LAYOUT_SCANNED) {
+#pragma unroll
+        for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
+            const int c = tid + k * EP_LAYOUT_THREADS;
+            if (c >= ncols) continue;
+            pre[k] = a.blk_cnt[(int64_t)b * a.cnt_stride + c];
+            tot[k] = a.col_total[c];
+        }
+    } else if (a.scan_mode == EP_LAYOUT_FOLDED) {
+        // ep_layout_count has finished and left plain counts: sum the rows before this workgroup's (and all
+        // rows) here.  A thread takes 4 adjacent columns (one 16-byte load a row) of every S-th row, EP_FOLD_DEPTH
+        // loads in flight (the rows come from memory: other XCDs wrote them); the S partial sums of a column
+        // meet in LDS (the per-wave counters are not in use yet).
+        const int W = a.cnt_stride, G = W >> 2;
+        int* s_fpre = s_we;                // [W]
+        int* s_ftot = s_we + W;            // [W]   (2 W <= NW * (E + R) ints)
+        for (int i = tid; i < 2 * W; i += blockDim.x) s_we[i] = 0;
+        __syncthreads();
+        const int nb = min(a.num_blocks, max(1, (num_rows + EP_TOKENS_PER_BLOCK - 1) / EP_TOKENS_PER_BLOCK));
+        const int S = G >= EP_LAYOUT_THREADS ? 1 : EP_LAYOUT_THREADS / G;
+        const int s0 = G >= EP_LAYOUT_THREADS ? 0 : tid / G;
+        if (s0 < S) {
+            for (int g = G >= EP_LAYOUT_THREADS ? tid : tid % G; g < G; g += EP_LAYOUT_THREADS) {
+                const u32x4* base = (const u32x4*)(a.blk_cnt + 4 * g);
+                const int64_t vstride = W >> 2;
+                int p0 = 0, p1 = 0, p2 = 0, p3 = 0, t0 = 0, t1 = 0, t2 = 0, t3 = 0;
+                for (int r = s0; r < nb; r += EP_FOLD_DEPTH * S) {
+                    u32x4 v[EP_FOLD_DEPTH];
+#pragma unroll
+                    for (int u = 0; u < EP_FOLD_DEPTH; ++u) {
+                        // unconditional loads (a row past the end re-reads the last one and is masked below), so
+                        // that all of them are in flight before the first is waited for
+                        v[u] = base[(int64_t)min(r + u * S, nb - 1) * vstride];
+                    }
+#pragma unroll
+                    for (int u = 0; u < EP_FOLD_DEPTH; ++u) {
+                        const int rr = r + u * S;
+                        const int mt = rr < nb ? -1 : 0, mp = rr < b ? -1 : 0;      // b <= nb - 1
+                        t0 += (int)v[u].x & mt; t1 += (int)v[u].y & mt; t2 += (int)v[u].z & mt; t3 += (int)v[u].w & mt;
+                        p0 += (int)v[u].x & mp; p1 += (int)v[u].y & mp; p2 += (int)v[u].z & mp; p3 += (int)v[u].w & mp;
+                    }
+                }
+                atomicAdd(&s_fpre[4 * g], p0); atomicAdd(&s_fpre[4 * g + 1], p1);
+                atomicAdd(&s_fpre[4 * g + 2], p2); atomicAdd(&s_fpre[4 * g + 3], p3);
+                atomicAdd(&s_ftot[4 * g], t0); atomicAdd(&s_ftot[4 * g + 1], t1);
+                atomicAdd(&s_ftot[4 * g + 2], t2); atomicAdd(&s_ftot[4 * g + 3], t3);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
+            const int c = tid + k * EP_LAYOUT_THREADS;
+            if (c >= ncols) continue;
+            pre[k] = s_fpre[c];
+            tot[k] = s_ftot[c];
+        }
+        __syncthreads();
+    }
+
     // ---- A: stage this block's keys, clear the per-wave counters ----
     for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
-    const int num_rows = layout_load_keys(a, s_key, s_rk, s_psum);
-    if (b > 0 && b * EP_TOKENS_PER_BLOCK >= num_rows) return;      // nothing to rank here, nothing to publish
+    layout_load_keys(a, s_key, s_rk, s_psum, num_rows);
     __syncthreads();
 
     // ---- B: per-wave counts: wave w owns entries [w*epw, (w+1)*epw) of this block's chunk ----
@@ -302,49 +368,28 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             const int e = s_key[idx];
             if (e >= 0) atomicAdd(&s_we[w * E + e], 1);
             const int mr = master_rank(s_rk, idx, K);
-            if (mr >= 0) atomicAdd(&s_wr[w * R + mr], 1);
+            if (mr >= 0) {
+                atomicAdd(&s_wr[w * R + mr], 1);
+                s_key[idx] = (short)(e | EP_KEY_MASTER);        // remembered for the ranking (only this thread reads it)
+            }
         }
     }
     __syncthreads();
 
-    // ---- C: counts of the blocks before this one (kept in registers) and totals over all blocks ----
-    int pre[EP_LAYOUT_MAX_COLS_PER_THREAD];
+    // ---- C: totals over all workgroups into LDS (one workgroup: its own per-wave counts are the totals) ----
 #pragma unroll
     for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
-        pre[k] = 0;
         const int c = tid + k * EP_LAYOUT_THREADS;
         if (c >= ncols) continue;
-        const bool is_expert = c < El;
-        const int col = is_expert ? lo + c : c - El;
-        const int stride = is_expert ? E : R;
-        int tot = 0;
-        if (a.scan_mode == EP_LAYOUT_SCANNED) {
-            pre[k] = (is_expert ? a.blk_expert_cnt : a.blk_rank_cnt)[(int64_t)b * stride + col];
-            tot = is_expert ? a.expert_total[col] : a.rank_total[col];
-        } else if (a.scan_mode == EP_LAYOUT_FOLDED) {
-            // ep_layout_count has finished: this block sums the counts of the blocks before it (and of all
-            // blocks) itself, one column per thread, consecutive threads on consecutive columns of a row
-            const int* base = (is_expert ? a.blk_expert_cnt : a.blk_rank_cnt) + col;
-            const int nb = min(a.num_blocks, max(1, (num_rows + EP_TOKENS_PER_BLOCK - 1) / EP_TOKENS_PER_BLOCK));
-            int before = 0;
-            int r = 0;
-            for (; r + 4 <= nb; r += 4) {
-                const int v0 = base[(int64_t)r * stride], v1 = base[(int64_t)(r + 1) * stride];
-                const int v2 = base[(int64_t)(r + 2) * stride], v3 = base[(int64_t)(r + 3) * stride];
-                before += (r < b ? v0 : 0) + (r + 1 < b ? v1 : 0) + (r + 2 < b ? v2 : 0) + (r + 3 < b ? v3 : 0);
-                tot += v0 + v1 + v2 + v3;
-            }
-            for (; r < nb; ++r) {
-                const int v = base[(int64_t)r * stride];
-                before += r < b ? v : 0;
-                tot += v;
-            }
-            pre[k] = before;
-        } else {
-            const int* wc = is_expert ? s_we + col : s_wr + col;
-            for (int i = 0; i < NW; ++i) tot += wc[i * stride];
+        if (a.scan_mode == EP_LAYOUT_SINGLE) {
+            const bool is_expert = c < El;
+            const int* wc = is_expert ? s_we + lo + c : s_wr + (c - El);
+            const int stride = is_expert ? E : R;
+            int t = 0;
+            for (int i = 0; i < NW; ++i) t += wc[i * stride];
+            tot[k] = t;
         }
-        s_tot[c] = tot;
+        s_tot[c] = tot[k];
     }
     __syncthreads();
 
@@ -433,10 +478,11 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     for (int rd = 0; rd < rounds; ++rd) {
         const int idx = w * epw + rd * WAVE + lane;
         const bool in = idx < n;
-        const int e = in ? s_key[idx] : -1;
+        const int key = in ? s_key[idx] : -1;
+        const int e = key < 0 ? -1 : key & (EP_KEY_MASTER - 1);
         const int le = e - lo;
         const bool local = e >= 0 && le >= 0 && le < El;
-        const int mr = in ? master_rank(s_rk, idx, K) : -1;
+        const int mr = (key >= 0 && (key & EP_KEY_MASTER)) ? s_rk[idx] : -1;
         const uint64_t pe = match_any(local ? e + 1 : 0, ebits);
         const uint64_t pr = match_any(mr + 1, rbits);
         int eslot = -1, rslot = -1;
@@ -474,8 +520,9 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             if (g >= num_rows || g >= a.rows_cap) continue;
             int master = -1;
             for (int j = 0; j < K; ++j) {
-                const int le = s_key[row * K + j] - lo;
-                if (le >= 0 && le < El) master = j;
+                const int key = s_key[row * K + j];
+                const int le = (key < 0 ? -1 : key & (EP_KEY_MASTER - 1)) - lo;
+                if (key >= 0 && le >= 0 && le < El) master = j;
             }
             const int64_t pr = recv_packed_row(s_psum, R, a.max_tokens, g);
             int* m = a.recv_src_metadata + (int64_t)g * (K + 2);
@@ -736,7 +783,7 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy_pac
     scatter_copy_body<true>(a);
 }
 
-template <bool HW, bool PACK>
+template <bool HW, bool PACK, bool LOADS = true>
 __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     if ((int)blockIdx.x >= a.num_row_blocks) {
         zero_padding_rows(a);
@@ -754,7 +801,8 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     const int v = part * WAVE + lane;
     const bool live = v < nvec;
     u32x4 d = {0u, 0u, 0u, 0u};
-    if (live) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
+    if (live && LOADS) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
+    if (!LOADS) d = u32x4{0x3f803f80u + (unsigned)v, 0x40004000u, 0xbf80bf80u, 0x3f003f00u};
     float f[8] = {bf16_lo(d.x), bf16_hi(d.x), bf16_lo(d.y), bf16_hi(d.y),
                   bf16_lo(d.z), bf16_hi(d.z), bf16_lo(d.w), bf16_hi(d.w)};
     unsigned mbits = 0u;
@@ -779,6 +827,12 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
 
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant(EpScatterArgs a) {
     scatter_quant_body<true, false>(a);
+}
+// Calibration: ep_scatter_quant with the loads of x taken out: the same tasks, the same stores to the same
+// slots (payload, scales, weights, metadata, zero padding), nothing read but the slot map.  Prices the
+// store pattern of the kernel by itself.
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_stores_only(EpScatterArgs a) {
+    scatter_quant_body<true, false, false>(a);
 }
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_sw(EpScatterArgs a) {
     scatter_quant_body<false, false>(a);
@@ -1079,6 +1133,24 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
 EP_COMBINE_KERNELS(, EP_COMBINE_FUSED)
 EP_COMBINE_KERNELS(_partial, EP_COMBINE_PARTIAL)
 EP_COMBINE_KERNELS(_final, EP_COMBINE_FINAL)
+
+// ------------------------------------------------------------------------------------------------
+// Calibration writes: what the memory system does with the simplest store patterns.  Workgroup b writes
+// one 4 KiB chunk with one 16-byte non-temporal store per thread; the chunks are visited in address order
+// (ep_calib_fill) or in a scrambled order (ep_calib_fill_shuffled: chunk = odd multiplier * b modulo the
+// chunk count, a power of two).
+// ------------------------------------------------------------------------------------------------
+extern "C" __global__ __launch_bounds__(256) void ep_calib_fill(EpCalibArgs a) {
+    u32x4* p = (u32x4*)a.dst + (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const u32x4 v = {a.value, a.value, a.value, a.value};
+    __builtin_nontemporal_store(v, p);
+}
+extern "C" __global__ __launch_bounds__(256) void ep_calib_fill_shuffled(EpCalibArgs a) {
+    const unsigned chunk = (blockIdx.x * 0x9E3779B1u) & (a.num_chunks - 1u);
+    u32x4* p = (u32x4*)a.dst + (int64_t)chunk * 256 + threadIdx.x;
+    const u32x4 v = {a.value, a.value, a.value, a.value};
+    __builtin_nontemporal_store(v, p);
+}
 
 // ------------------------------------------------------------------------------------------------
 // Self-test: hardware e4m3fn conversion against the integer conversion over a range of fp32 bit

@@ -114,13 +114,14 @@ struct Kernels {
     hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw, sf_transpose;
     hipFunction_t scatter_copy_pack, scatter_quant_pack, scatter_quant_sw_pack;
     hipFunction_t combine[3][5];     // [mode][generic, k2, k4, k6, k8]
-    hipFunction_t fp8_selftest;
+    hipFunction_t fp8_selftest, scatter_quant_stores_only, calib_fill, calib_fill_shuffled;
     int device = -1;
 };
 
 std::mutex g_mutex;
 Kernels g_k;
 bool g_fp8_hw = true;
+bool g_stores_only = false;     // calibration: the fused-quantising copy kernel runs without its loads of x
 int g_fold_max_blocks = 256;    // up to this many layout workgroups the slot assignment sums the block counts itself
 
 std::string library_dir() {
@@ -161,6 +162,9 @@ void load_kernels(const char* dir) {
         for (int k = 0; k < 5; ++k)
             get(g_k.combine[mode][k], (std::string("ep_combine") + modes[mode] + ks[k]).c_str());
     get(g_k.fp8_selftest, "ep_fp8_selftest");
+    get(g_k.scatter_quant_stores_only, "ep_scatter_quant_stores_only");
+    get(g_k.calib_fill, "ep_calib_fill");
+    get(g_k.calib_fill_shuffled, "ep_calib_fill_shuffled");
     g_k.module = m;
 }
 
@@ -349,6 +353,20 @@ void ep_host_f32_to_e4m3fn(const float* src, uint8_t* dst, int64_t n) {
 }
 
 void ep_set_fp8_hw_convert(int enable) { g_fp8_hw = enable != 0; }
+
+void ep_set_calibration_stores_only(int enable) { g_stores_only = enable != 0; }
+
+int ep_calibrate_fill(void* dst, int64_t num_bytes, int shuffled, unsigned value, void* stream) {
+    return guarded([&] {
+        load_kernels(nullptr);
+        EP_HOST_ASSERT(dst != nullptr and ((uintptr_t)dst & 15) == 0);
+        EP_HOST_ASSERT(num_bytes > 0 and num_bytes % 4096 == 0 and num_bytes / 4096 <= INT32_MAX);
+        const unsigned chunks = (unsigned)(num_bytes / 4096);
+        EP_HOST_ASSERT(not shuffled or (chunks & (chunks - 1)) == 0);       // the scrambled order needs a power of two
+        EpCalibArgs ca = {dst, chunks, value};
+        launch(shuffled ? g_k.calib_fill_shuffled : g_k.calib_fill, chunks, 256, 0, stream, ca);
+    });
+}
 
 int ep_fp8_selftest(uint64_t first, uint64_t count, float limit, uint64_t out[2]) {
     return guarded([&] {
@@ -660,10 +678,9 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             return p;
         };
         EpLayoutArgs la{};
-        la.expert_total = carve(E);
-        la.rank_total = carve(R);
-        la.blk_expert_cnt = carve((int64_t)num_blocks * E);
-        la.blk_rank_cnt = carve((int64_t)num_blocks * R);
+        la.cnt_stride = (int)align_up(E / R + R, 4);
+        la.col_total = carve(la.cnt_stride);
+        la.blk_cnt = carve((int64_t)num_blocks * la.cnt_stride);
         if (R == 1) {
             la.slot_map = carve((int64_t)num_tokens * K);
             la.recv_tok = carve(a.num_max_tokens_per_rank);
@@ -771,10 +788,9 @@ int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
             return p;
         };
         EpLayoutArgs la{};
-        la.expert_total = carve(E);
-        la.rank_total = carve(R);
-        la.blk_expert_cnt = carve((int64_t)num_blocks * E);
-        la.blk_rank_cnt = carve((int64_t)num_blocks * R);
+        la.cnt_stride = (int)align_up(E / R + R, 4);
+        la.col_total = carve(la.cnt_stride);
+        la.blk_cnt = carve((int64_t)num_blocks * la.cnt_stride);
         EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= b->workspace_bytes and "layout scratch of the receive stream fits the workspace");
         la.recv_mode = 1;
         la.num_tokens = (int)rows_bound;
@@ -981,6 +997,7 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         const unsigned grid = (unsigned)sa.num_row_blocks + pad_blocks;
         if (grid > 0) {
             hipFunction_t fn = quantise_here ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
+            if (quantise_here and g_stores_only) fn = g_k.scatter_quant_stores_only;
             launch(fn, grid, EP_ROW_THREADS, 0, a.stream, sa);
         }
         if (sf_columns and num_expanded > 0) {
