@@ -57,7 +57,7 @@ struct EpLayoutArgs {
     int* col_total;               // [cnt_stride]  column totals (written by ep_layout_scan)
     int cnt_stride;               // El + R rounded up to a multiple of 4 ints
     int* slot_map;                // [T, K]  expanded slot of (t, j) if its expert is local, else -1
-    int* recv_tok;                // [max_tokens]  receive-stream row -> local token index
+    int* tok_row;                 // [T]  token -> its row of the receive stream (written for received tokens only)
     // handle tensors (device)
     int* dst_buffer_slot_idx;     // [T, K]
     int* dst_gsge_idx;            // [T, K]
@@ -85,8 +85,8 @@ struct EpScatterArgs {
     const void* sf;               // input scale factors (prequantised FP8) or null
     const float* topk_weights;    // [T, K] or null
     const int* slot_map;          // [T, K]   (non-cached)
-    const int* recv_tok;          // [N]      (non-cached)
-    const int* num_recv_ptr;      // device scalar: psum_rank[R-1]
+    const int* tok_row;           // [T]      (non-cached)
+    const int* num_recv_ptr;      // device scalar: psum_rank[R-1]  (modes whose rows are the receive stream)
     int* recv_src_metadata;       // [N, K+2]  written (non-cached) / read (cached)
     void* recv_x;                 // [N_exp, hidden] out
     void* recv_sf;                // out or null
@@ -102,7 +102,7 @@ struct EpScatterArgs {
     int cached;                   // slots come from recv_src_metadata
     int num_sf_packs;             // 2-byte packs per row (prequantised) ; fused: hidden/128 floats
     int num_local_experts, expert_alignment;
-    int reserved0;
+    int num_meta_rows;            // rows recv_src_metadata holds
     int num_row_blocks;           // blocks [0, num_row_blocks) copy rows, the rest zero padding
     int num_tokens;               // T: bound of the token indices a row may name
     int num_parts;                // column parts per row; a wave task is (row, part)
@@ -125,6 +125,7 @@ struct EpScatterArgs {
     int num_ranks;
     int pack_sf_off;              // byte offset of the scales inside a packed row (pack mode)
     int vecs_per_lane;            // verbatim kernel: 16-byte vectors a lane moves per task (1..4)
+    int rows_are_tokens;          // cached expand: every token was received, so row i of the receive stream is token i
 };
 
 // recv_sf layouts: rows of scales, or columns of scales whose stride is the row count of recv_sf

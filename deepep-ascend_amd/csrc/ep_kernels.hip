@@ -504,7 +504,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
                 a.dst_gsge_idx[g] = -1;             // every copy is local: no transport descriptors
                 if (!a.send_only) {
                     a.slot_map[g] = eslot;
-                    if (mr == a.rank_idx && rslot < a.max_tokens) a.recv_tok[rslot] = b * EP_TOKENS_PER_BLOCK + idx / K;
+                    if (mr == a.rank_idx) a.tok_row[b * EP_TOKENS_PER_BLOCK + idx / K] = rslot;
                 }
             }
         }
@@ -607,8 +607,9 @@ __device__ __forceinline__ char* out_sf_of(const EpScatterArgs& a, char* rows) {
 
 // A wave task is (row, column part).  Resolves the row's token, its source row and its destination
 // rows; the task of part 0 also writes the row's small items.  Three modes:
-//   EP_SCATTER_EXPAND  rows of the receive stream, payload read from x[token]; destinations are the
-//                      expanded slots; part 0 writes the metadata row (non-cached) and the gate weights
+//   EP_SCATTER_EXPAND  rows are tokens (non-cached: slots from the slot map) or rows of the receive stream
+//                      (cached: slots and token from the metadata row), payload read from x[token]; destinations
+//                      are the expanded slots; part 0 writes the metadata row (non-cached) and the gate weights
 //   EP_SCATTER_PACK    rows are tokens; destinations are rows of the partition-major regions
 //                      (partition * max_tokens + slot of dst_buffer_slot_idx); part 0 writes the packed
 //                      metadata [all K topk_idx | all K weights | src_token_global_idx] into each of them
@@ -657,6 +658,7 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
     if (a.mode == EP_SCATTER_REGION) {
         // the metadata rows are complete before this kernel runs: written by the receive-side layout, or cached
         const int v = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
+        if (i >= *a.num_recv_ptr) return false;          // (checked after the row's own load has been issued)
         if (lane < K && v >= 0 && v < a.num_out_rows) myslot = v;
         c.src_row = region_row_of_stream(a.psum_rank, a.num_ranks, a.max_tokens, i);
         if (part == 0 && a.recv_topk_weights != nullptr && myslot >= 0)
@@ -666,18 +668,22 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
         return true;
     }
     if (!a.cached) {
-        t = a.recv_tok[i];
-        if (t < 0 || t >= a.num_tokens) return false;
+        // the tasks walk the tokens (nothing has to be looked up before the row of x can be fetched); the row of
+        // the receive stream a token became is only needed for its metadata row
+        t = i;
         if (lane < K) myslot = a.slot_map[(int64_t)t * K + lane];
+        const uint64_t vm = __ballot(myslot >= 0);
+        if (vm == 0) return false;                       // a token nobody receives
         if (part == 0) {
-            const uint64_t vm = __ballot(myslot >= 0);
-            const int master = vm == 0 ? -1 : 63 - __builtin_clzll(vm);
+            const int row = a.tok_row[t];
+            const int master = 63 - __builtin_clzll(vm);
             // [slot_0 .. slot_{K-1}, src_token_global_idx, last local j]  (dispatch_copy_epilogue.hpp:514-522)
             const int v = lane < K ? myslot : (lane == K ? a.rank_idx * a.max_tokens + t : master);
-            if (lane < K + 2) a.recv_src_metadata[(int64_t)i * (K + 2) + lane] = v;
+            if (lane < K + 2 && row >= 0 && row < a.num_meta_rows) a.recv_src_metadata[(int64_t)row * (K + 2) + lane] = v;
         }
     } else {
         const int v = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
+        if (i >= *a.num_recv_ptr) return false;          // (checked after the row's own load has been issued)
         if (lane < K) myslot = v;
         t = readlane(v, K) - a.rank_idx * a.max_tokens;
         if (t < 0 || t >= a.num_tokens) return false;
@@ -689,6 +695,14 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
     c.t = t;
     c.myslot = myslot;
     return true;
+}
+
+// Source row of task row i if it is known before the prologue has run, else -1.
+template <bool PACK>
+__device__ __forceinline__ int64_t scatter_guess_source_row(const EpScatterArgs& a, int i) {
+    if (PACK) return i;                                            // rows are tokens
+    if (a.mode == EP_SCATTER_EXPAND && (!a.cached || a.rows_are_tokens)) return i;
+    return -1;
 }
 
 // The padding rows of an expert, [psum[e], align(psum[e], A)), are one contiguous span of each output:
@@ -733,21 +747,34 @@ __device__ __forceinline__ void scatter_copy_body(const EpScatterArgs& a) {
     const int lane = lane_id();
     const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
     const int i = task / a.num_parts, part = task - i * a.num_parts;
-    const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
-    if (i >= n) return;
-    RowCtx c;
-    if (!scatter_row_prologue<PACK>(a, i, part, c)) return;
+    if (i >= a.num_rows_bound) return;
     const int K = a.num_topk;
     const int nvec = (int)(a.copy_bytes >> 4);
     // a task moves vecs_per_lane KiB of the row: 1 where a row fans out to several slots, more where
     // nearly every row has a single destination and the set-up above would outweigh the copy
     const int U = a.vecs_per_lane;
     u32x4 d[4];
+    // Where the source row of a task is known up front (tokens are walked, or every token was received so that
+    // row i of the receive stream is token i), its payload is fetched while the prologue looks up the slots;
+    // a prologue that names another row after all fetches again.
+    const int64_t guess = scatter_guess_source_row<PACK>(a, i);
+    if (guess >= 0) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int v = (part * U + u) * WAVE + lane;
-        if (u < U && v < nvec)
-            d[u] = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
+        for (int u = 0; u < 4; ++u) {
+            const int v = (part * U + u) * WAVE + lane;
+            if (u < U && v < nvec)
+                d[u] = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + guess * a.x_row_bytes) + v);
+        }
+    }
+    RowCtx c;
+    if (!scatter_row_prologue<PACK>(a, i, part, c)) return;
+    if (c.src_row != guess) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int v = (part * U + u) * WAVE + lane;
+            if (u < U && v < nvec)
+                d[u] = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
+        }
     }
     for (int j = 0; j < K; ++j) {
         const int s = readlane(c.myslot, j);
@@ -792,16 +819,19 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     const int lane = lane_id();
     const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
     const int i = task / a.num_parts, part = task - i * a.num_parts;
-    const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
-    if (i >= n) return;
-    RowCtx c;
-    if (!scatter_row_prologue<PACK>(a, i, part, c)) return;
+    if (i >= a.num_rows_bound) return;
     const int K = a.num_topk;
     const int nvec = a.hidden >> 3;                      // 16-byte vectors of 8 BF16
     const int v = part * WAVE + lane;
     const bool live = v < nvec;
     u32x4 d = {0u, 0u, 0u, 0u};
-    if (live && LOADS) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
+    // the payload is fetched while the prologue looks up the slots wherever the source row is known up front
+    const int64_t guess = scatter_guess_source_row<PACK>(a, i);
+    if (live && LOADS && guess >= 0) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + guess * a.x_row_bytes) + v);
+    RowCtx c;
+    if (!scatter_row_prologue<PACK>(a, i, part, c)) return;
+    if (live && LOADS && c.src_row != guess)
+        d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + c.src_row * a.x_row_bytes) + v);
     if (!LOADS) d = u32x4{0x3f803f80u + (unsigned)v, 0x40004000u, 0xbf80bf80u, 0x3f003f00u};
     float f[8] = {bf16_lo(d.x), bf16_hi(d.x), bf16_lo(d.y), bf16_hi(d.y),
                   bf16_lo(d.z), bf16_hi(d.z), bf16_lo(d.w), bf16_hi(d.w)};
@@ -978,8 +1008,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     const int K = KT > 0 ? KT : a.num_topk;
     const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
     const int i = task / a.num_parts, part = task - i * a.num_parts;
-    const int n = a.num_recv_ptr != nullptr ? min(*a.num_recv_ptr, a.num_rows_bound) : a.num_rows_bound;
-    if (i >= n) return;
+    if (i >= a.num_rows_bound) return;
 
     int myslot = -1, t, group = 0, src_rank = 0;
     if (MODE == EP_COMBINE_FINAL) {
@@ -997,6 +1026,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
         if (master) myslot = (a.num_ranks < K ? r : lane) * a.max_tokens + t;
     } else {
         const int mv = lane < K + 2 ? a.recv_src_metadata[(int64_t)i * (K + 2) + lane] : -1;
+        if (i >= *a.num_recv_ptr) return;                // (checked after the row's own load has been issued)
         if (lane < K && mv >= 0 && mv < a.num_in_rows) myslot = mv;
         const int src = readlane(mv, K);                        // source partition * max_tokens + its token
         if (MODE == EP_COMBINE_PARTIAL) {
@@ -1032,7 +1062,8 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
             if (lane < K) ((unsigned*)a.combined_topk_weights)[(int64_t)t * K + lane] = acc;
         }
     } else {
-        if (a.expanded_weights != nullptr && myslot >= 0) myw = a.expanded_weights[myslot];
+        const bool need_w = part == 0 || (MODE == EP_COMBINE_FUSED && a.weighted);
+        if (need_w && a.expanded_weights != nullptr && myslot >= 0) myw = a.expanded_weights[myslot];
         if (part == 0 && lane < K) {
             if (MODE == EP_COMBINE_FUSED && a.combined_topk_weights != nullptr)
                 a.combined_topk_weights[(int64_t)t * K + lane] = myw;
@@ -1045,8 +1076,76 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     const bool has_bias = a.bias_0 != nullptr || a.bias_1 != nullptr;
     const int v0 = part * 2 * WAVE + lane, v1 = v0 + WAVE;
     const bool live0 = v0 < nvec, live1 = v1 < nvec;
+    const bool weighted = MODE == EP_COMBINE_FUSED && a.weighted;
+    // the gate weights are scattered 4-byte loads: only the task that carries them back (part 0) or multiplies
+    // by them has read them; the other tasks hold zeros
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    if (KT > 0) {
+        // Every load of the task is issued before the first add: the biases of the token (token-side reduce), then
+        // both 16-byte vectors of every input row.  The two vectors are then reduced one after the other, which
+        // keeps the live registers at the loaded vectors plus one accumulator (72 VGPRs at K = 6: seven waves a SIMD).
+        u32x4 b0[2], b1[2], d0[KT > 0 ? KT : 1], d1[KT > 0 ? KT : 1];
+        int nb = 0;
+        if (MODE == EP_COMBINE_FINAL) {
+            const void* biases[2] = {a.bias_0, a.bias_1};
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                if (biases[b] == nullptr) continue;
+                const u32x4* bp = (const u32x4*)biases[b] + (int64_t)t * nvec;
+                b0[nb] = live0 ? bp[v0] : zero;
+                b1[nb] = live1 ? bp[v1] : zero;
+                ++nb;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < KT; ++j) {
+            const int s = readlane(myslot, j);
+            if (s < 0) continue;
+            if (live0) d0[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + v0);
+            if (live1) d1[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + v1);
+        }
+        // inputs in order: b0, b1, then the rows in ascending position; zero inputs -> zeros, one input -> verbatim
+        // copy, more -> one rounding of the fp32 sum (a weighted single row is a product: rounded as well)
+        auto reduce = [&](const u32x4* bias, const u32x4* d) -> u32x4 {
+            float acc[8], g[8];
+            u32x4 first = zero;
+            int nin = 0;
+            for (int b = 0; b < nb; ++b) {
+                unpack8(bias[b], g);
+                if (nin == 0) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; first = bias[b]; }
+                else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
+                ++nin;
+            }
+#pragma unroll
+            for (int j = 0; j < KT; ++j) {
+                const int s = readlane(myslot, j);
+                if (s < 0) continue;
+                unpack8(d[j], g);
+                if (weighted) {
+                    const float wj = __int_as_float(readlane(__float_as_int(myw), j));
+                    for (int q = 0; q < 8; ++q) g[q] = g[q] * wj;
+                }
+                if (nin == 0) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; first = d[j]; }
+                else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
+                ++nin;
+            }
+            if (nin >= 2 || (weighted && nin == 1)) return pack8(acc);
+            return first;
+        };
+        if (live0) {
+            u32x4 res = reduce(b0, d0);
+            if (MODE == EP_COMBINE_FUSED && has_bias) res = add_biases(a, t, v0, true, res);
+            stream_store<EP_COMBINE_ST_POL>(out + v0, res);
+        }
+        if (live1) {
+            u32x4 res = reduce(b1, d1);
+            if (MODE == EP_COMBINE_FUSED && has_bias) res = add_biases(a, t, v1, true, res);
+            stream_store<EP_COMBINE_ST_POL>(out + v1, res);
+        }
+        return;
+    }
     float acc0[8], acc1[8];
-    u32x4 res0 = {0u, 0u, 0u, 0u}, res1 = {0u, 0u, 0u, 0u};
+    u32x4 res0 = zero, res1 = zero;
     int nin = 0;                                              // inputs accumulated so far
     if (MODE == EP_COMBINE_FINAL) {
         const void* biases[2] = {a.bias_0, a.bias_1};
@@ -1054,7 +1153,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
         for (int b = 0; b < 2; ++b) {
             if (biases[b] == nullptr) continue;
             const u32x4* bp = (const u32x4*)biases[b] + (int64_t)t * nvec;
-            u32x4 e0 = {0u, 0u, 0u, 0u}, e1 = {0u, 0u, 0u, 0u};
+            u32x4 e0 = zero, e1 = zero;
             if (live0) e0 = bp[v0];
             if (live1) e1 = bp[v1];
             float g0[8], g1[8];
@@ -1065,51 +1164,25 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
             ++nin;
         }
     }
-    if (KT > 0) {
-        u32x4 d0[KT > 0 ? KT : 1], d1[KT > 0 ? KT : 1];
-#pragma unroll
-        for (int j = 0; j < KT; ++j) {
-            const int s = readlane(myslot, j);
-            if (s < 0) continue;
-            if (live0) d0[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + v0);
-            if (live1) d1[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + v1);
+    for (int j = 0; j < K; ++j) {
+        const int s = readlane(myslot, j);
+        if (s < 0) continue;
+        u32x4 e0 = zero, e1 = zero;
+        if (live0) e0 = __builtin_nontemporal_load(y + (int64_t)s * yvec + v0);
+        if (live1) e1 = __builtin_nontemporal_load(y + (int64_t)s * yvec + v1);
+        float g0[8], g1[8];
+        unpack8(e0, g0);
+        unpack8(e1, g1);
+        if (weighted) {
+            const float wj = __int_as_float(readlane(__float_as_int(myw), j));
+            for (int q = 0; q < 8; ++q) { g0[q] = g0[q] * wj; g1[q] = g1[q] * wj; }
         }
-#pragma unroll
-        for (int j = 0; j < KT; ++j) {
-            const int s = readlane(myslot, j);
-            if (s < 0) continue;
-            float g0[8], g1[8];
-            unpack8(d0[j], g0);
-            unpack8(d1[j], g1);
-            if (MODE == EP_COMBINE_FUSED && a.weighted) {
-                const float wj = __int_as_float(readlane(__float_as_int(myw), j));
-                for (int q = 0; q < 8; ++q) { g0[q] = g0[q] * wj; g1[q] = g1[q] * wj; }
-            }
-            if (nin == 0) { for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; } res0 = d0[j]; res1 = d1[j]; }
-            else { for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; } }
-            ++nin;
-        }
-    } else {
-        for (int j = 0; j < K; ++j) {
-            const int s = readlane(myslot, j);
-            if (s < 0) continue;
-            u32x4 e0 = {0u, 0u, 0u, 0u}, e1 = {0u, 0u, 0u, 0u};
-            if (live0) e0 = __builtin_nontemporal_load(y + (int64_t)s * yvec + v0);
-            if (live1) e1 = __builtin_nontemporal_load(y + (int64_t)s * yvec + v1);
-            float g0[8], g1[8];
-            unpack8(e0, g0);
-            unpack8(e1, g1);
-            if (MODE == EP_COMBINE_FUSED && a.weighted) {
-                const float wj = __int_as_float(readlane(__float_as_int(myw), j));
-                for (int q = 0; q < 8; ++q) { g0[q] = g0[q] * wj; g1[q] = g1[q] * wj; }
-            }
-            if (nin == 0) { for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; } res0 = e0; res1 = e1; }
-            else { for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; } }
-            ++nin;
-        }
+        if (nin == 0) { for (int q = 0; q < 8; ++q) { acc0[q] = g0[q]; acc1[q] = g1[q]; } res0 = e0; res1 = e1; }
+        else { for (int q = 0; q < 8; ++q) { acc0[q] = acc0[q] + g0[q]; acc1[q] = acc1[q] + g1[q]; } }
+        ++nin;
     }
     // zero inputs -> zeros, one input -> verbatim copy, more -> one rounding of the fp32 sum
-    if (nin >= 2 || (MODE == EP_COMBINE_FUSED && a.weighted && nvalid == 1)) {
+    if (nin >= 2 || (weighted && nvalid == 1)) {
         res0 = pack8(acc0);
         res1 = pack8(acc1);
     }

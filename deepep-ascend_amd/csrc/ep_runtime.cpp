@@ -223,7 +223,7 @@ struct ep_buffer {
         int64_t stamp = 0;
         int num_tokens = 0, num_topk = 0, num_experts = 0, alignment = 0, max_tokens = 0;
         int* slot_map = nullptr;
-        int* recv_tok = nullptr;
+        int* tok_row = nullptr;
         bool notified = false;
         bool recv_done = false;     // more than one partition: the receive-side layout has been enqueued
     } last;
@@ -683,7 +683,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         la.blk_cnt = carve((int64_t)num_blocks * la.cnt_stride);
         if (R == 1) {
             la.slot_map = carve((int64_t)num_tokens * K);
-            la.recv_tok = carve(a.num_max_tokens_per_rank);
+            la.tok_row = carve(num_tokens);
         }
         if (b->is_static and off * (int64_t)sizeof(int) > b->workspace_bytes)
             throw EpError{format("Assertion exception (%s:%d): the layout scratch of %d tokens x top-%d over %d experts (%lld bytes) "
@@ -728,7 +728,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
         b->last.alignment = a.expert_alignment;
         b->last.max_tokens = a.num_max_tokens_per_rank;
         b->last.slot_map = la.slot_map;
-        b->last.recv_tok = la.recv_tok;
+        b->last.tok_row = la.tok_row;
         b->last.notified = do_cpu_sync and R == 1;
         b->last.recv_done = false;
     });
@@ -929,7 +929,7 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         EpScatterArgs sa{};
         sa.topk_weights = (const float*)a.topk_weights.data;
         sa.slot_map = b->last.slot_map;
-        sa.recv_tok = b->last.recv_tok;
+        sa.tok_row = b->last.tok_row;
         sa.num_recv_ptr = (const int*)a.psum_num_recv_tokens_per_rank.data + (R - 1);
         sa.recv_src_metadata = (int*)a.recv_src_metadata.data;
         sa.recv_x = a.recv_x.data;
@@ -944,6 +944,7 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         // never walk past the rows the metadata tensor holds
         sa.num_rows_bound = (int)std::min<int64_t>(b->recv_rows_bound(num_tokens, a.num_max_tokens_per_rank),
                                                    a.recv_src_metadata.size[0]);
+        sa.num_meta_rows = (int)std::min<int64_t>(a.recv_src_metadata.size[0], INT32_MAX);
         sa.num_tokens = num_tokens;
         sa.rank_idx = b->rank_idx;
         sa.max_tokens = a.num_max_tokens_per_rank;
@@ -955,6 +956,13 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         if (R == 1) {
             // one partition: the packed intermediate is skipped, rows come straight from x
             sa.mode = EP_SCATTER_EXPAND;
+            if (not cached_mode) {
+                // the tasks walk the tokens, not the receive stream: no device count bounds them
+                sa.num_recv_ptr = nullptr;
+                sa.num_rows_bound = num_tokens;
+            }
+            // a cached handle that holds one metadata row per token: row i is token i (the rows ascend with the token)
+            sa.rows_are_tokens = cached_mode and a.recv_src_metadata.size[0] == num_tokens ? 1 : 0;
             sa.x = a.x.data;
             sa.sf = a.sf.data;
             sa.x_row_bytes = (int64_t)hidden * elem_size(a.x.dtype);
