@@ -365,6 +365,8 @@ def main():
                     help='also time pure writes of the copy kernel\'s byte count: 4 KiB chunks in address order '
                          '(ep_calib_fill), in scrambled order (ep_calib_fill_shuffled), torch\'s fill, and the copy '
                          'kernel with its loads taken out (ep_scatter_quant_stores_only)')
+    ap.add_argument('--combine-blocks-per-cu', type=int, default=None,
+                    help='tuning: workgroups of a combine kernel a CU holds at once (library default 4; 0: no cap)')
     ap.add_argument('--samples', type=int, default=50, help='isolated, cache-flushed launches per kernel')
     args = ap.parse_args()
     if args.graph:
@@ -375,6 +377,8 @@ def main():
         sys.exit(2)
 
     import deep_ep
+    if args.combine_blocks_per_cu is not None:
+        deep_ep._C.set_combine_blocks_per_cu(args.combine_blocks_per_cu)
     T, H, E, K, A, fp8 = WORKLOADS[args.workload]
     dev = torch.device('cuda', 0)
     torch.cuda.set_device(dev)

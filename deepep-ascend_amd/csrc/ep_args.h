@@ -172,6 +172,7 @@ struct EpCombineArgs {
     // owner-side reduce: the partial of a row goes to the combine buffer of the partition its token came from
     char* const* peer_arenas;
     int64_t buffer_off;
+    int whole_rows;               // owner-side reduce: a task is a whole row (num_parts == 1), not a 1024-channel part
 };
 
 // Hardware vs integer e4m3fn conversion over fp32 bit patterns [first, first+count).

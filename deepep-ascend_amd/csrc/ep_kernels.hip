@@ -1074,9 +1074,29 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
 
     u32x4* out = (u32x4*)out_row;
     const bool has_bias = a.bias_0 != nullptr || a.bias_1 != nullptr;
-    const int v0 = part * 2 * WAVE + lane, v1 = v0 + WAVE;
-    const bool live0 = v0 < nvec, live1 = v1 < nvec;
     const bool weighted = MODE == EP_COMBINE_FUSED && a.weighted;
+    // Owner side with whole rows per task: a received row mostly has a single slot among this partition's few
+    // experts, and its partial is then that row verbatim: up to 16 vectors a lane in flight, no arithmetic.
+    if (MODE == EP_COMBINE_PARTIAL && a.whole_rows && nvalid == 1) {
+        const int s1 = readlane(myslot, __builtin_ctzll(__ballot(myslot >= 0)));
+        const u32x4* src = y + (int64_t)s1 * yvec;
+        for (int vb = lane; vb < nvec; vb += 16 * WAVE) {
+            u32x4 d[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                if (vb + u * WAVE < nvec) d[u] = __builtin_nontemporal_load(src + vb + u * WAVE);
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                if (vb + u * WAVE < nvec) stream_store<EP_COMBINE_ST_POL>(out + vb + u * WAVE, d[u]);
+        }
+        return;
+    }
+    // a task is one 1024-channel part of its row, or (owner side, whole rows) all of them in turn
+    const bool whole = MODE == EP_COMBINE_PARTIAL && a.whole_rows;
+    const int part_end = whole ? (nvec + 2 * WAVE - 1) / (2 * WAVE) : part + 1;
+    for (int cp = whole ? 0 : part; cp < part_end; ++cp) {
+    const int v0 = cp * 2 * WAVE + lane, v1 = v0 + WAVE;
+    const bool live0 = v0 < nvec, live1 = v1 < nvec;
     // the gate weights are scattered 4-byte loads: only the task that carries them back (part 0) or multiplies
     // by them has read them; the other tasks hold zeros
     const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -1142,7 +1162,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
             if (MODE == EP_COMBINE_FUSED && has_bias) res = add_biases(a, t, v1, true, res);
             stream_store<EP_COMBINE_ST_POL>(out + v1, res);
         }
-        return;
+        continue;
     }
     float acc0[8], acc1[8];
     u32x4 res0 = zero, res1 = zero;
@@ -1193,6 +1213,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     if (live1) {
         if (MODE == EP_COMBINE_FUSED && has_bias) res1 = add_biases(a, t, v1, true, res1);
         stream_store<EP_COMBINE_ST_POL>(out + v1, res1);
+    }
     }
 }
 

@@ -122,6 +122,17 @@ std::mutex g_mutex;
 Kernels g_k;
 bool g_fp8_hw = true;
 bool g_stores_only = false;     // calibration: the fused-quantising copy kernel runs without its loads of x
+// Workgroups of the single-partition combine kernel a CU holds at once, enforced through an unused dynamic LDS
+// allocation (0: no cap, the registers decide: 5 to 7).  Measured at the headline shape (top-6, 12 row fetches of
+// 1 KiB a wave): 7 a CU 291 us, 5: 287, 4: 275-278, 3: 282, 2: 320; top-8 at 4096 tokens and the two-phase
+// kernels of the partitioned path do not react to it.
+int g_combine_blocks_per_cu = 4;
+constexpr unsigned kLdsBytesPerCu = 160 * 1024;
+unsigned combine_lds_cap() {
+    if (g_combine_blocks_per_cu <= 0) return 0;
+    const unsigned share = kLdsBytesPerCu / (unsigned)g_combine_blocks_per_cu;
+    return std::min(64u * 1024u, share - 1024u);       // n of them fit a CU, n + 1 do not
+}
 int g_fold_max_blocks = 256;    // up to this many layout workgroups the slot assignment sums the block counts itself
 
 std::string library_dir() {
@@ -740,6 +751,8 @@ int64_t ep_dispatch_stamp(ep_buffer_t* b) {
 
 void ep_set_layout_fold_max_blocks(int num_blocks) { g_fold_max_blocks = num_blocks; }
 
+void ep_set_combine_blocks_per_cu(int num_blocks) { g_combine_blocks_per_cu = num_blocks; }
+
 int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
     return guarded([&] {
         EP_HOST_ASSERT(pa != nullptr);
@@ -1109,6 +1122,9 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             ca.peer_arenas = b->peer_table();
             ca.buffer_off = b->workspace_bytes;
             ca.out_row_bytes = combine_token;
+            // a received row mostly has one slot among a partition's few experts: whole rows per wave task
+            ca.whole_rows = 1;
+            ca.num_parts = 1;
             ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
             if (ca.num_row_blocks == 0) return;
             launch(g_k.combine[EP_COMBINE_PARTIAL][kidx], (unsigned)ca.num_row_blocks, EP_ROW_THREADS, 0, a.stream, ca);
@@ -1138,7 +1154,7 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
             const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(num_combined_tokens, EP_ROW_THREADS);
             if (grid == 0) return;
-            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, 0, a.stream, ca);
+            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, combine_lds_cap(), a.stream, ca);
         } else {
             check_peers(b, [&](const ep_buffer& p) { return p.num_partials >= b->num_partials; },
                         "its owner-side reduce (phase 0) comes before any token-side reduce");

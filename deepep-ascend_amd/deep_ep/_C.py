@@ -108,6 +108,7 @@ _ep_dispatch_epi = _sig('ep_dispatch_epilogue_launch', ctypes.c_int, ctypes.c_vo
                         ctypes.POINTER(_DispatchEpilogueArgs))
 _ep_stamp = _sig('ep_dispatch_stamp', ctypes.c_int64, ctypes.c_void_p)
 _ep_set_fold = _sig('ep_set_layout_fold_max_blocks', None, ctypes.c_int)
+_ep_set_combine_cap = _sig('ep_set_combine_blocks_per_cu', None, ctypes.c_int)
 _ep_dispatch_static = _sig('ep_dispatch_static_launch', ctypes.c_int, ctypes.POINTER(_DispatchArgs),
                            ctypes.POINTER(_DispatchEpilogueArgs))
 _ep_combine = _sig('ep_combine_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_CombineArgs), ctypes.c_int)
@@ -252,6 +253,11 @@ def calibrate_fill(dst: torch.Tensor, shuffled: bool = False, value: int = 0) ->
 def set_calibration_stores_only(enable: bool) -> None:
     """Calibration: the fused-quantising copy kernel runs without its loads of x (outputs are garbage)."""
     _ep_set_stores_only(int(enable))
+
+
+def set_combine_blocks_per_cu(num_blocks: int) -> None:
+    """Tuning: workgroups of a combine kernel a compute unit holds at once (0: no cap).  Results do not depend on it."""
+    _ep_set_combine_cap(int(num_blocks))
 
 
 def set_layout_fold_max_blocks(num_blocks: int) -> None:

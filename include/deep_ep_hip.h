@@ -176,6 +176,10 @@ int64_t ep_dispatch_stamp(ep_buffer_t* buf);
  * not depend on it. */
 void ep_set_layout_fold_max_blocks(int num_blocks);
 
+/* Tuning: workgroups (of 4 waves) of the single-partition combine kernel that a compute unit holds at once;
+ * 0 lifts the cap (default 4).  Results do not depend on it. */
+void ep_set_combine_blocks_per_cu(int num_blocks);
+
 /* More than one partition, non-cached dispatch: the receive side of launch_dispatch and the slot
  * assignment of the copy epilogue (impls/ep/dispatch.hpp:469-545,
  * impls/ep/dispatch_copy_epilogue.hpp:130-174,397-423,471-488,514-522).  Walks the rows that
