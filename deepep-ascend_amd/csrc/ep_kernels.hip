@@ -2,16 +2,18 @@
 // `hipcc --genco` and launched by the host runtime through hipModuleLaunchKernel.
 //
 // Kernels (all HBM-bound, no MFMA):
-//   ep_layout_count / ep_layout_scan / ep_layout_assign   stable counting sort of the (token, slot)
+//   ep_layout_count / ep_layout_assign (/ ep_layout_scan)  stable counting sort of the (token, slot)
 //       entries by destination partition and by local expert -> every handle tensor; with several
 //       partitions once on the send side (slots in the destinations' regions) and once on the receive
-//       side (slots of the rows that arrived)
-//   ep_scatter_copy / ep_scatter_quant                     receive-stream row -> its expanded slots
+//       side (slots of the rows that arrived).  Two launches up to a few hundred workgroups (the
+//       assignment sums the histograms of the workgroups before it itself), three beyond.
+//   ep_scatter_copy / ep_scatter_quant                     token (or receive-stream row) -> its expanded slots
 //   ep_scatter_copy_pack / ep_scatter_quant_pack           token -> one packed row per destination partition
 //   ep_sf_transpose                                        scale rows -> scale columns
 //   ep_combine_k<K> / ep_combine_generic                   K-way gather + fp32 reduce back to token order
 //   ep_combine_partial_* / ep_combine_final_*              the same reduce in its owner-side and token-side halves
 //   ep_fp8_selftest                                        hardware vs integer e4m3fn conversion
+//   ep_calib_fill / ep_calib_fill_shuffled / ep_scatter_quant_stores_only   write-path calibration for benchmarks
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -261,8 +263,8 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
 // (impls/ep/dispatch.hpp:469-545) and, when asked, the host count page.
 //
 // Where the counts of the other blocks come from (a.scan_mode):
-//   EP_LAYOUT_SCANNED  ep_layout_scan left exclusive prefixes in blk_*_cnt and totals in *_total
-//   EP_LAYOUT_FOLDED   ep_layout_count left plain counts in blk_*_cnt: every block sums the rows before it
+//   EP_LAYOUT_SCANNED  ep_layout_scan left exclusive prefixes in blk_cnt and totals in col_total
+//   EP_LAYOUT_FOLDED   ep_layout_count left plain counts in blk_cnt: every block sums the rows before it
 //                      itself (cheaper than a launch of its own up to a few hundred blocks)
 //   EP_LAYOUT_SINGLE   one block owns every token: nothing ran before, its own LDS counts are the totals
 // Only the local experts and the partitions need prefixes: slots of other experts are never used.
@@ -533,7 +535,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
 }
 
 // ------------------------------------------------------------------------------------------------
-// Scatter (dispatch copy epilogue): one receive-stream row per wave.
+// Scatter (dispatch copy epilogue): a wave task is one column part of one row (a token, or a row of the receive stream).
 // Reference semantics: impls/ep/dispatch_copy_epilogue.hpp:450-545 (expand), :547-620 (zero padding).
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_lo(unsigned int u) { return __uint_as_float(u << 16); }

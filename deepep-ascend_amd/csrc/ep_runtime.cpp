@@ -1012,7 +1012,9 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
             1, quantise_here ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024 * sa.vecs_per_lane));
         sa.num_row_blocks = (int)ceil_div((int64_t)sa.num_rows_bound * sa.num_parts, EP_ROWS_PER_BLOCK);
         EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0);
-        // an expert has at most alignment - 1 padding rows: about one workgroup per 8 of them
+        // an expert has at most alignment - 1 padding rows: about one workgroup per 8 of them (measured: 16 a
+        // expert at alignment 128 and 32 or 64 give the same time; one per 4 KiB chunk, 223 a expert, is 10-20 %
+        // slower: every workgroup first waits for the expert's row count)
         sa.pad_blocks_per_expert = std::max(1, std::min(EP_MAX_PAD_BLOCKS_PER_EXPERT, a.expert_alignment / 8));
         const unsigned pad_blocks = a.do_zero_padding ? (unsigned)(El * sa.pad_blocks_per_expert) : 0u;
         const unsigned grid = (unsigned)sa.num_row_blocks + pad_blocks;
@@ -1122,9 +1124,12 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             ca.peer_arenas = b->peer_table();
             ca.buffer_off = b->workspace_bytes;
             ca.out_row_bytes = combine_token;
-            // a received row mostly has one slot among a partition's few experts: whole rows per wave task
-            ca.whole_rows = 1;
-            ca.num_parts = 1;
+            // a received row mostly has one slot among a partition's few experts: whole rows per wave task once
+            // there are enough rows to fill the machine that way (a few thousand rows are spread part by part)
+            if (ca.num_rows_bound >= 16384) {
+                ca.whole_rows = 1;
+                ca.num_parts = 1;
+            }
             ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
             if (ca.num_row_blocks == 0) return;
             launch(g_k.combine[EP_COMBINE_PARTIAL][kidx], (unsigned)ca.num_row_blocks, EP_ROW_THREADS, 0, a.stream, ca);
