@@ -169,8 +169,11 @@ def calibrate_write(deep_ep, timed, n, dispatch, handle, T, H, K, n_valid, n_rec
 
     entry('ep_calib_fill', med(timed(lambda: deep_ep._C.calibrate_fill(area[:seq_bytes]), n)), seq_bytes,
           '4 KiB per workgroup, one 16-byte non-temporal store per thread, address order')
-    entry('ep_calib_fill_shuffled', med(timed(lambda: deep_ep._C.calibrate_fill(area, shuffled=True), n)), pow2_bytes,
+    entry('ep_calib_fill_shuffled', med(timed(lambda: deep_ep._C.calibrate_fill(area, shuffled=1), n)), pow2_bytes,
           'the same chunks in a scrambled order')
+    for unit in (4, 16, 256):                                         # 16 KiB, 64 KiB, 1 MiB
+        entry(f'ep_calib_fill_shuffled_{unit * 4}KiB', med(timed(lambda: deep_ep._C.calibrate_fill(area, shuffled=unit), n)),
+              pow2_bytes, f'runs of {unit} chunks ({unit * 4} KiB) kept together, the runs scrambled')
     entry('torch_fill', med(timed(lambda: area[:seq_bytes].zero_(), n)), seq_bytes, 'torch zero_() of the same bytes')
     deep_ep._C.set_calibration_stores_only(True)
     try:

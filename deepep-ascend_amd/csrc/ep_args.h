@@ -188,4 +188,6 @@ struct EpCalibArgs {
     void* dst;
     unsigned num_chunks;
     unsigned value;
+    unsigned unit_chunks;         // scrambled order: consecutive chunks that stay together (a power of two)
+    unsigned pad;
 };

@@ -1233,8 +1233,8 @@ EP_COMBINE_KERNELS(_final, EP_COMBINE_FINAL)
 // ------------------------------------------------------------------------------------------------
 // Calibration writes: what the memory system does with the simplest store patterns.  Workgroup b writes
 // one 4 KiB chunk with one 16-byte non-temporal store per thread; the chunks are visited in address order
-// (ep_calib_fill) or in a scrambled order (ep_calib_fill_shuffled: chunk = odd multiplier * b modulo the
-// chunk count, a power of two).
+// (ep_calib_fill) or in a scrambled order (ep_calib_fill_shuffled: runs of unit_chunks chunks stay together,
+// run = odd multiplier * index modulo the number of runs, a power of two).
 // ------------------------------------------------------------------------------------------------
 extern "C" __global__ __launch_bounds__(256) void ep_calib_fill(EpCalibArgs a) {
     u32x4* p = (u32x4*)a.dst + (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -1242,7 +1242,10 @@ extern "C" __global__ __launch_bounds__(256) void ep_calib_fill(EpCalibArgs a) {
     __builtin_nontemporal_store(v, p);
 }
 extern "C" __global__ __launch_bounds__(256) void ep_calib_fill_shuffled(EpCalibArgs a) {
-    const unsigned chunk = (blockIdx.x * 0x9E3779B1u) & (a.num_chunks - 1u);
+    // units of unit_chunks consecutive chunks keep their inner order; the units are scrambled
+    const unsigned unit = blockIdx.x / a.unit_chunks, in_unit = blockIdx.x - unit * a.unit_chunks;
+    const unsigned num_units = a.num_chunks / a.unit_chunks;
+    const unsigned chunk = ((unit * 0x9E3779B1u) & (num_units - 1u)) * a.unit_chunks + in_unit;
     u32x4* p = (u32x4*)a.dst + (int64_t)chunk * 256 + threadIdx.x;
     const u32x4 v = {a.value, a.value, a.value, a.value};
     __builtin_nontemporal_store(v, p);

@@ -368,13 +368,15 @@ void ep_set_fp8_hw_convert(int enable) { g_fp8_hw = enable != 0; }
 void ep_set_calibration_stores_only(int enable) { g_stores_only = enable != 0; }
 
 int ep_calibrate_fill(void* dst, int64_t num_bytes, int shuffled, unsigned value, void* stream) {
+    // shuffled: 0 = address order; n > 0 = runs of n chunks (a power of two) in a scrambled order
     return guarded([&] {
         load_kernels(nullptr);
         EP_HOST_ASSERT(dst != nullptr and ((uintptr_t)dst & 15) == 0);
         EP_HOST_ASSERT(num_bytes > 0 and num_bytes % 4096 == 0 and num_bytes / 4096 <= INT32_MAX);
         const unsigned chunks = (unsigned)(num_bytes / 4096);
-        EP_HOST_ASSERT(not shuffled or (chunks & (chunks - 1)) == 0);       // the scrambled order needs a power of two
-        EpCalibArgs ca = {dst, chunks, value};
+        EP_HOST_ASSERT(shuffled >= 0 and (shuffled & (shuffled - 1)) == 0);
+        EP_HOST_ASSERT(not shuffled or ((chunks & (chunks - 1)) == 0 and (unsigned)shuffled <= chunks));   // powers of two
+        EpCalibArgs ca = {dst, chunks, value, (unsigned)std::max(1, shuffled), 0u};
         launch(shuffled ? g_k.calib_fill_shuffled : g_k.calib_fill, chunks, 256, 0, stream, ca);
     });
 }

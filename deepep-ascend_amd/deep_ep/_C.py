@@ -243,9 +243,9 @@ def set_fp8_hw_convert(enable: bool) -> None:
     _ep_set_hw(int(enable))
 
 
-def calibrate_fill(dst: torch.Tensor, shuffled: bool = False, value: int = 0) -> None:
-    """Calibration write over the whole of `dst` (a multiple of 4 KiB; a power-of-two number of 4 KiB chunks
-    when shuffled) on the current stream: one 4 KiB chunk per workgroup, in address or scrambled order."""
+def calibrate_fill(dst: torch.Tensor, shuffled: int = 0, value: int = 0) -> None:
+    """Calibration write over the whole of `dst` (a multiple of 4 KiB) on the current stream: one 4 KiB chunk per
+    workgroup, in address order, or with runs of `shuffled` chunks in a scrambled order (powers of two)."""
     init_jit()
     _check(_ep_calib_fill(dst.data_ptr(), dst.numel() * dst.element_size(), int(shuffled), value, _stream()))
 

@@ -81,8 +81,8 @@ void ep_set_fp8_hw_convert(int enable);
 
 /* Calibration of the store path, for benchmarks (no counterpart in the reference).
  * ep_calibrate_fill: num_bytes / 4096 workgroups each write one 4 KiB chunk of dst with one 16-byte
- * non-temporal store per thread, in address order or (shuffled; the chunk count must then be a power of
- * two) in a scrambled order.  ep_set_calibration_stores_only(1): from then on the fused-quantising copy
+ * non-temporal store per thread, in address order (shuffled = 0) or with runs of `shuffled` consecutive
+ * chunks in a scrambled order (shuffled and the chunk count powers of two).  ep_set_calibration_stores_only(1): from then on the fused-quantising copy
  * kernel of ep_dispatch_epilogue_launch runs without its loads of x (same tasks, same stores to the same
  * slots, arbitrary payload): the price of the kernel's store pattern alone.  Outputs are garbage while it
  * is on. */
@@ -259,7 +259,11 @@ typedef struct ep_combine_args {
 /* Validates like EPBuffer::combine (csrc/buffers/ep.hpp:426-481).  Replaces launch_combine and
  * launch_combine_reduce_epilogue (csrc/kernels/ep/combine.hpp:18-112); `phase` selects which
  * half of the reference's two launches is enqueued: 0 = owner-side reduce, 1 = token-side
- * reduce into combined_x.  With one partition the whole reduction runs in phase 1. */
+ * reduce into combined_x.  With one partition the whole reduction runs in phase 1.  Phase 1 of a
+ * buffer that is one partition of several reads, for every token, one partial per destination
+ * partition from this buffer's combine region: in a connected node the peers' phase 0 put them there;
+ * a partition used alone (not connected) holds only its own partials after phase 0, the caller
+ * places the others (what a transport would deliver) before phase 1. */
 int ep_combine_launch(ep_buffer_t* buf, const ep_combine_args_t* args, int phase);
 
 #ifdef __cplusplus
