@@ -255,6 +255,43 @@ def test_cached_dispatch_replays_layout():
     buf.destroy()
 
 
+@pytest.mark.parametrize('unrouted', [(), (0,), (3, 77, 199)])
+@pytest.mark.parametrize('do_cpu_sync', [True, False])
+@pytest.mark.parametrize('fused', [False, True])
+def test_cached_replay_whatever_rows_map_to_tokens(unrouted, do_cpu_sync, fused):
+    """A cached replay fetches the payload of "row i = token i" ahead of the metadata row when the handle holds one
+    metadata row per token, and fetches again when the row names another token.  Every token received (the guess is
+    right), tokens nobody receives with exact counts (fewer rows than tokens: no guess), and the same with a handle of
+    worst-case sizes (as many rows as tokens: the guess is wrong behind the first such token)."""
+    T, H, E, K, A = 200, 512, 32, 4, 16
+    topk, w = make_routing(T, E, K, seed=15)
+    for t in unrouted:
+        topk[t] = -1
+        w[t] = 0
+    lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, T)
+    assert lay['num_recv_tokens'] == T - len(unrouted)
+    buf = _buffer(T, H, K, fp8=fused)
+    kw = dict(do_expand=True, do_zero_padding=True, fused_fp8_quant=fused)
+    _, _, _, handle, _ = buf.dispatch(make_tokens(T, H, seed=1).to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV),
+                                      num_experts=E, num_max_tokens_per_rank=T, expert_alignment=A,
+                                      do_cpu_sync=do_cpu_sync, **kw)
+    assert handle.recv_src_metadata.size(0) == (lay['num_recv_tokens'] if do_cpu_sync else T)
+    x2 = make_tokens(T, H, seed=2, outliers=True)
+    recv, _, rw, _, _ = buf.dispatch(x2.to(DEV), topk_weights=w.to(DEV), handle=handle, **kw)
+    torch.cuda.synchronize()
+    ne = lay['num_expanded_tokens']
+    if fused:
+        q, sf = O.quantise(x2)
+        ex, es, ew = O.rank_share_dispatch(q.numpy(), sf.numpy().view(np.uint32), w.numpy(), lay)
+        assert np.array_equal(recv[0].view(torch.uint8).cpu().numpy()[:ne], ex)
+        assert np.array_equal(recv[1].cpu().numpy().view(np.uint32)[:ne], es)
+    else:
+        ex, _, ew = O.rank_share_dispatch(bf16_bits(x2), None, w.numpy(), lay)
+        assert np.array_equal(bf16_bits(recv)[:ne], ex)
+    assert np.array_equal(rw.cpu().numpy().view(np.uint32)[:ne], ew.view(np.uint32))
+    buf.destroy()
+
+
 def test_dispatch_without_host_sync_uses_worst_case_sizes():
     T, H, E, K, A = 96, 256, 16, 4, 8
     x = make_tokens(T, H, seed=2)
