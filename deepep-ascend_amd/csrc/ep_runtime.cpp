@@ -273,7 +273,7 @@ void launch_layout(EpLayoutArgs& la, int num_blocks, void* stream) {
     if (la.scan_mode != EP_LAYOUT_SINGLE)
         launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, layout_count_lds(E, R, K), stream, la);
     if (la.scan_mode == EP_LAYOUT_SCANNED)
-        launch(g_k.layout_scan, (unsigned)ceil_div(E + R, 16), EP_SCAN_THREADS, 0, stream, la);
+        launch(g_k.layout_scan, (unsigned)ceil_div(la.cnt_stride, 16), EP_SCAN_THREADS, 0, stream, la);
     launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, stream, la);
 }
 
@@ -1200,6 +1200,7 @@ ep_buffer* static_view_of_current_device() {
     int dev = -1;
     HIP_CHECK(hipGetDevice(&dev));
     EP_HOST_ASSERT(dev >= 0 and dev < kMaxDevices);
+    EP_HOST_ASSERT(dev == g_k.device and "the kernels were loaded on another device");
     std::lock_guard<std::mutex> lock(g_static_mutex);
     ep_buffer* v = &g_static_view[dev];
     if (v->arena == nullptr) {
