@@ -181,3 +181,17 @@ def test_bench_byte_formulas_give_the_headline_figures():
     assert bench.combine_bytes(T, H, K, T * K, T, 0, True) == 1646264320
     assert bench.dispatch_bytes(4096, H, 8, 4096 * 8, 4096, False, False) == 529432576      # BF16 top-8
     assert bench.WORKLOADS['c3_headline'] == (T, H, 256, K, 128, True)
+
+
+def test_committed_traffic_summary_belongs_to_the_kernel_sources():
+    """bench.py reports HBM traffic from the committed counter summary only while that summary was taken from
+    the kernel sources in the tree (its kernel_source_sha256 line): a kernel change needs a fresh counter run."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location('bench_module_traffic', os.path.join(ROOT, 'bench.py'))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    traffic, source = bench.measured_traffic('c3_headline')
+    assert source.endswith('headline_dispatch_combine_hbm_traffic.txt'), source
+    # measured traffic = algorithmic bytes (+ the zero padding the copy kernel also writes), nothing re-read
+    assert 1.0 <= traffic['ep_scatter_quant'] / (964427776 + 115495936) < 1.02
+    assert 1.0 <= traffic['ep_combine_k6'] / 1646264320 < 1.02
