@@ -889,6 +889,18 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         EP_HOST_ASSERT(a.num_experts % R == 0);
         const int El = a.num_experts / R;
         const bool fused = a.fused_fp8_quant != 0;
+        // the same input contract as ep_dispatch_launch: this entry point may be called on its own
+        if (present(a.sf)) {
+            EP_HOST_ASSERT(not fused and a.x.dtype == EP_DTYPE_FP8_E4M3);
+            EP_HOST_ASSERT(a.sf.ndim == 2 and a.sf.size[0] == num_tokens and elem_size(a.sf.dtype) == 2);
+            EP_HOST_ASSERT(a.sf.stride[0] == 1 or a.sf.stride[1] == 1);
+            EP_HOST_ASSERT(a.sf.stride[0] <= INT32_MAX and a.sf.stride[1] <= INT32_MAX);
+        } else {
+            EP_HOST_ASSERT(a.x.dtype == EP_DTYPE_BF16);
+        }
+        EP_HOST_ASSERT(not fused or (hidden % 8 == 0 and hidden <= 16384));
+        EP_HOST_ASSERT(a.num_max_tokens_per_rank > 0 and num_tokens <= a.num_max_tokens_per_rank);
+        EP_HOST_ASSERT(a.expert_alignment > 0);
         EP_HOST_ASSERT(present(a.recv_x) and a.recv_x.ndim == 2 and a.recv_x.size[1] == hidden);
         EP_HOST_ASSERT(contiguous(a.recv_x));
         EP_HOST_ASSERT(a.recv_x.dtype == (fused ? (int)EP_DTYPE_FP8_E4M3 : a.x.dtype));
@@ -920,14 +932,17 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         if (present(a.topk_weights)) {
             EP_HOST_ASSERT(present(a.recv_topk_weights) and a.recv_topk_weights.ndim == 1);
             EP_HOST_ASSERT(a.recv_topk_weights.size[0] == num_expanded and a.recv_topk_weights.dtype == EP_DTYPE_F32);
-            EP_HOST_ASSERT(a.topk_weights.size[0] == num_tokens and a.topk_weights.size[1] == K);
+            EP_HOST_ASSERT(a.topk_weights.ndim == 2 and a.topk_weights.size[0] == num_tokens and a.topk_weights.size[1] == K);
+            EP_HOST_ASSERT(contiguous(a.topk_weights) and a.topk_weights.dtype == EP_DTYPE_F32);
+            EP_HOST_ASSERT(contiguous(a.recv_topk_weights));
         }
         EP_HOST_ASSERT(present(a.recv_src_metadata) and a.recv_src_metadata.ndim == 2);
         EP_HOST_ASSERT(a.recv_src_metadata.size[1] == K + 2);
         EP_HOST_ASSERT(contiguous(a.recv_src_metadata));
         EP_HOST_ASSERT(a.recv_src_metadata.dtype == EP_DTYPE_I32);
-        EP_HOST_ASSERT(present(a.psum_num_recv_tokens_per_rank) and a.psum_num_recv_tokens_per_rank.size[0] == R);
-        EP_HOST_ASSERT(present(a.psum_num_recv_tokens_per_expert) and a.psum_num_recv_tokens_per_expert.size[0] == El);
+        for (const ep_tensor_t* ps : {&a.psum_num_recv_tokens_per_rank, &a.psum_num_recv_tokens_per_expert})
+            EP_HOST_ASSERT(present(*ps) and ps->ndim == 1 and contiguous(*ps) and ps->dtype == EP_DTYPE_I32);
+        EP_HOST_ASSERT(a.psum_num_recv_tokens_per_rank.size[0] == R and a.psum_num_recv_tokens_per_expert.size[0] == El);
         if (not cached_mode) {
             EP_HOST_ASSERT(b->last.valid and "the copy epilogue follows its own dispatch launch");
             // the slot map and the receive order live in the workspace, which every dispatch launch overwrites
@@ -1012,8 +1027,10 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         sa.vecs_per_lane = sa.mode == EP_SCATTER_REGION ? 4 : 1;
         sa.num_parts = (int)std::max<int64_t>(
             1, quantise_here ? ceil_div(hidden, 512) : ceil_div(sa.copy_bytes, 1024 * sa.vecs_per_lane));
-        sa.num_row_blocks = (int)ceil_div((int64_t)sa.num_rows_bound * sa.num_parts, EP_ROWS_PER_BLOCK);
-        EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0);
+        const int64_t row_blocks = ceil_div((int64_t)sa.num_rows_bound * sa.num_parts, EP_ROWS_PER_BLOCK);
+        EP_HOST_ASSERT(row_blocks <= INT32_MAX / 2);
+        sa.num_row_blocks = (int)row_blocks;
+        EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0 and sa.x_row_bytes % 16 == 0);
         // an expert has at most alignment - 1 padding rows: about one workgroup per 8 of them (measured: 16 a
         // expert at alignment 128 and 32 or 64 give the same time; one per 4 KiB chunk, 223 a expert, is 10-20 %
         // slower: every workgroup first waits for the expert's row count)
