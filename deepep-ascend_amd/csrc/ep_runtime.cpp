@@ -1030,7 +1030,8 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         const int64_t row_blocks = ceil_div((int64_t)sa.num_rows_bound * sa.num_parts, EP_ROWS_PER_BLOCK);
         EP_HOST_ASSERT(row_blocks <= INT32_MAX / 2);
         sa.num_row_blocks = (int)row_blocks;
-        EP_HOST_ASSERT(sa.out_row_bytes % 16 == 0 and sa.x_row_bytes % 16 == 0);
+        // rows are read in 16-byte vectors; the verbatim kernel writes them so, the quantising one 8 bytes a lane
+        EP_HOST_ASSERT(sa.x_row_bytes % 16 == 0 and sa.out_row_bytes % (quantise_here ? 8 : 16) == 0);
         // an expert has at most alignment - 1 padding rows: about one workgroup per 8 of them (measured: 16 a
         // expert at alignment 128 and 32 or 64 give the same time; one per 4 KiB chunk, 223 a expert, is 10-20 %
         // slower: every workgroup first waits for the expert's row count)
