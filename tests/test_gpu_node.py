@@ -129,7 +129,8 @@ def test_node_dispatch_combine(R, max_tokens, H, E, K, A, masked, mode, do_cpu_s
         assert np.array_equal(rx.view(torch.uint8).cpu().numpy().reshape(rx.size(0), -1)[:ne], want[r]['x'])
         if rsf is not None:
             assert rsf.stride() == ((1, rsf.size(0)) if col_major else (rsf.size(1), 1))
-            assert np.array_equal(rsf.contiguous().view(torch.uint8).cpu().numpy().reshape(rsf.size(0), -1)[:ne],
+            # (numpy makes the copy row-major: torch calls a single column of any stride contiguous already)
+            assert np.array_equal(np.ascontiguousarray(rsf.cpu().numpy()).view(np.uint8).reshape(rsf.size(0), -1)[:ne],
                                   want[r]['sf'])
         assert np.array_equal(rw.cpu().numpy().view(np.uint32)[:ne], want[r]['w'].view(np.uint32))
         handles.append(handle)
@@ -162,7 +163,7 @@ def test_node_dispatch_combine(R, max_tokens, H, E, K, A, masked, mode, do_cpu_s
         rx2, rsf2 = recv2 if isinstance(recv2, tuple) else (recv2, None)
         assert np.array_equal(rx2.view(torch.uint8).cpu().numpy().reshape(rx2.size(0), -1)[:ne], want2[r]['x'])
         if rsf2 is not None:
-            assert np.array_equal(rsf2.contiguous().view(torch.uint8).cpu().numpy().reshape(rsf2.size(0), -1)[:ne],
+            assert np.array_equal(np.ascontiguousarray(rsf2.cpu().numpy()).view(np.uint8).reshape(rsf2.size(0), -1)[:ne],
                                   want2[r]['sf'])
         assert np.array_equal(rw2.cpu().numpy().view(np.uint32)[:ne], want2[r]['w'].view(np.uint32))
 

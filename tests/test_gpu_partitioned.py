@@ -88,7 +88,7 @@ def test_partitioned_dispatch(T, H, E, K, A, R, rank, masked, mode):
     got_x = rx.view(torch.uint8).cpu().numpy().reshape(rx.size(0), -1)
     assert np.array_equal(got_x, ex)
     if sfb:
-        assert np.array_equal(rsf.contiguous().view(torch.uint8).cpu().numpy().reshape(rsf.size(0), -1), es)
+        assert np.array_equal(np.ascontiguousarray(rsf.cpu().numpy()).view(np.uint8).reshape(rsf.size(0), -1), es)
     assert np.array_equal(rw.cpu().numpy().view(np.uint32), ew.view(np.uint32))
 
     # cached replay: new payload and weights through the same layout
