@@ -459,8 +459,8 @@ def main():
         loop_dispatch = sorted(m[0].elapsed_time(m[1]) * 1e3 for m in marks)
         loop_combine = sorted(m[1].elapsed_time(m[2]) * 1e3 for m in marks)
 
-    # Isolated samples: the copy kernel alone is what a cached dispatch enqueues.  Ten untimed launches, then
-    # --samples timed ones; before each a 1 GiB scratch buffer is rewritten, so no sample finds its inputs in
+    # Isolated samples: each kernel alone (the copy kernel as the epilogue of a deferred dispatch, and again as
+    # what a cached dispatch enqueues).  Ten untimed launches, then --samples timed ones; before each a 1 GiB scratch buffer is rewritten, so no sample finds its inputs in
     # the L2 or the memory-side cache (the reference's benchmark does the same: tests/ep/test_ep.py:79-80,
     # 415-421).  The median is reported (the mean beside it).
     scratch = None if args.no_flush else torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -478,8 +478,26 @@ def main():
         torch.cuda.synchronize()
         return sorted(a.elapsed_time(b) * 1e3 for a, b in evs)      # microseconds
 
+    def timed_copy_kernel(n, warm=10):
+        # The copy kernel of a non-cached dispatch by itself: the layout kernels of a deferred dispatch run in
+        # front of the bracket, its epilogue (the copy kernel, then the host's read of the counts) inside.
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for k in range(warm + n):
+            if scratch is not None:
+                scratch.zero_()
+            ev = buf.dispatch(xg, topk_idx=tg, topk_weights=wg, do_cpu_sync=not args.no_cpu_sync,
+                              async_with_compute_stream=True, defer_epilogue=True, **kw)
+            if k >= warm:
+                evs[k - warm][0].record()
+            ev.current_stream_wait()
+            if k >= warm:
+                evs[k - warm][1].record()
+        torch.cuda.synchronize()
+        return sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
+
     n_k = args.samples
-    t_scatter = timed(lambda: dispatch(handle), n_k)
+    t_scatter = timed_copy_kernel(n_k)
+    t_scatter_cached = timed(lambda: dispatch(handle), n_k)
     t_combine = timed(lambda: buf.combine(y, handle, topk_weights=recv_w), n_k)
     t_dispatch_full = timed(lambda: dispatch(), n_k)
     # the layout kernels alone: a deferred dispatch enqueues them and returns; its copy epilogue runs outside the
@@ -528,6 +546,8 @@ def main():
     kernels = [roof(scatter_name, b_d, t_scatter), roof(f'ep_combine_k{K}', b_c, t_combine)]
     for k in kernels:
         k['sampled'] = 'isolated launches' + ('' if args.no_flush else ', caches flushed before each')
+    kernels[0]['sampled'] += '; the epilogue of a deferred non-cached dispatch (its layout kernels in front of the bracket)'
+    kernels[0]['us_cached_replay'] = round(med(t_scatter_cached), 2)
     # The dominant kernel, priced on its launches inside the timed region (event to event on the launch
     # stream: the kernel plus the gap to its predecessor).
     if loop_combine is not None:
