@@ -63,6 +63,7 @@ def measured_traffic(workload):
 WORKLOADS = {
     # name: (T, H, E, K, A, fp8)
     'c3_headline': (16384, 7168, 256, 6, 128, True),
+    'c3_prequantised': (16384, 7168, 256, 6, 128, True),   # the caller quantises: dispatch of (FP8 rows, scale packs)
     'c2_bf16_top8': (4096, 7168, 256, 8, 128, False),
     'c1_small': (128, 256, 8, 2, 1, False),
     'c4_decode_zipf': (128, 7168, 256, 8, 128, True),
@@ -400,16 +401,21 @@ def main():
         return
     x, topk, w = make_inputs(T, H, E, K)
     xg, tg, wg = x.to(dev), topk.to(dev), w.to(dev)
+    fused = fp8 and args.workload != 'c3_prequantised'
+    if fp8 and not fused:
+        # the drop-in form of the reference: the caller's quantiser, scales handed over as 2-byte packs
+        xq, xs = deep_ep.utils.math.per_token_cast_to_fp8(xg)
+        xg = (xq, xs.view(torch.int16))
     buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K,
                            use_fp8_dispatch=fp8, explicitly_destroy=True)
     kw = dict(num_experts=E, num_max_tokens_per_rank=T, expert_alignment=A, do_expand=True, do_zero_padding=True,
-              fused_fp8_quant=fp8)
+              fused_fp8_quant=fused)
 
     def dispatch(handle=None):
         if handle is None:
             return buf.dispatch(xg, topk_idx=tg, topk_weights=wg, do_cpu_sync=not args.no_cpu_sync, **kw)
         return buf.dispatch(xg, topk_weights=wg, handle=handle, do_expand=True, do_zero_padding=True,
-                            fused_fp8_quant=fp8)
+                            fused_fp8_quant=fused)
 
     recv, _, recv_w, handle, _ = dispatch()
     n_exp = (recv[0] if fp8 else recv).size(0)
@@ -418,7 +424,7 @@ def main():
     n_valid = int(handle.num_unaligned_recv_tokens_per_expert.sum().item())
     n_recv = int(handle.psum_num_recv_tokens_per_rank[-1].item())
     n_exp_exact = int(handle.psum_num_recv_tokens_per_expert[-1].item() + A - 1) // A * A
-    b_d = dispatch_bytes(T, H, K, n_valid, n_recv, fp8, fp8)
+    b_d = dispatch_bytes(T, H, K, n_valid, n_recv, fp8, fused)
     b_c = combine_bytes(T, H, K, n_valid, n_recv, 0, True)
     pad_bytes = (n_exp_exact - n_valid) * (H * (1 if fp8 else 2) + ((H // 128) * 4 if fp8 else 0) + 4)
 
@@ -542,7 +548,7 @@ def main():
                 'us_mean': round(avg(samples), 2), 'us_min': round(samples[0], 2), 'samples': len(samples),
                 'bytes': nbytes}
 
-    scatter_name = 'ep_scatter_quant' if fp8 else 'ep_scatter_copy'
+    scatter_name = 'ep_scatter_quant' if fused else 'ep_scatter_copy'
     kernels = [roof(scatter_name, b_d, t_scatter), roof(f'ep_combine_k{K}', b_c, t_combine)]
     for k in kernels:
         k['sampled'] = 'isolated launches' + ('' if args.no_flush else ', caches flushed before each')
@@ -576,7 +582,7 @@ def main():
         'data': 'synthetic',
         'config': {'workload': args.workload, 'tokens': T, 'hidden': H, 'experts': E, 'topk': K,
                    'expert_alignment': A, 'partitions': 1, 'dispatch': 'fused bf16->fp8 e4m3 + per-128 fp32 scales'
-                   if fp8 else 'bf16', 'combine': 'bf16, fp32 accumulate, weights carried back, no bias',
+                   if fused else ('fp8 e4m3 rows + per-128 fp32 scales quantised by the caller' if fp8 else 'bf16'), 'combine': 'bf16, fp32 accumulate, weights carried back, no bias',
                    'do_zero_padding': True, 'do_cpu_sync': not args.no_cpu_sync, 'hip_graph': bool(args.graph),
                    'cache_flush_between_kernel_samples': not args.no_flush,
                    'num_valid_rows': n_valid, 'num_expanded_rows': n_exp_exact},
@@ -598,7 +604,7 @@ def main():
             'scatter_gbs_incl_padding': round((b_d + pad_bytes) / us_scatter / 1e3, 1),
         },
     }
-    if args.calibrate_write and fp8:
+    if args.calibrate_write and fused:
         out['write_calibration'] = calibrate_write(deep_ep, timed, n_k, dispatch, handle, T, H, K, n_valid, n_recv,
                                                    pad_bytes, dev, us_scatter)
     if not args.no_cpu_baseline:
