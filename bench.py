@@ -98,22 +98,34 @@ def make_inputs(T, H, E, K, seed=0):
 
 def cpu_small_case():
     """The reference's CPU-runnable case (128 tokens x 256, 8 experts, top-2, alignment 1, BF16 dispatch then
-    combine of the dispatched rows) on the host cores: median of 5 passes of the oracle."""
+    combine of the dispatched rows) on the host cores: median of 20 passes of the oracle after 3 untimed ones."""
     from oracle import ep_oracle as O
     T, H, E, K, A, _ = WORKLOADS['c1_small']
     x, topk, w = make_inputs(T, H, E, K, seed=1)
     ts = []
-    for _ in range(5):
+    for k in range(3 + 20):             # three untimed passes, then the median of twenty
         t0 = time.perf_counter()
         lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, T)
         rx, _, rw = O.rank_share_dispatch(x.view(torch.int16).numpy(), None, w.numpy(), lay)
         O.combine_fast(torch.from_numpy(rx).view(torch.bfloat16), torch.from_numpy(rw), lay['recv_src_metadata'], T, K)
-        ts.append(time.perf_counter() - t0)
+        if k >= 3:
+            ts.append(time.perf_counter() - t0)
     n_valid = int(lay['num_unaligned_recv_tokens_per_expert'].sum())
     nbytes = dispatch_bytes(T, H, K, n_valid, lay['num_recv_tokens'], False, False) + \
         combine_bytes(T, H, K, n_valid, lay['num_recv_tokens'], 0, True)
     med = sorted(ts)[len(ts) // 2]
     return {'workload': 'c1_small', 'ms': round(med * 1e3, 3), 'gbs': round(nbytes / med / 1e9, 3)}
+
+
+def cpu_model():
+    try:
+        with open('/proc/cpuinfo') as f:
+            for line in f:
+                if line.startswith('model name'):
+                    return line.split(':', 1)[1].strip()
+    except OSError:
+        pass
+    return 'unknown'
 
 
 def cpu_baseline(H, E, K, A, fp8, sample_tokens, budget_s=12.0, max_passes=16):
@@ -149,6 +161,7 @@ def cpu_baseline(H, E, K, A, fp8, sample_tokens, budget_s=12.0, max_passes=16):
                        combine_bytes(sample_tokens, H, K, n_valid, n_recv, 0, True))
     secs = t_dispatch + t_combine
     return {'value': round(nbytes / secs / 1e9, 3), 'unit': 'GB/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+            'cpu_model': cpu_model(),
             'sample': f'{passes} passes over {sample_tokens} tokens of the workload: dispatch {t_dispatch:.2f} s + '
                       f'combine {t_combine:.2f} s of numpy/torch-CPU oracle (os.cpu_count()={os.cpu_count()})',
             'small_case': cpu_small_case()}
