@@ -383,7 +383,7 @@ def main():
                          '(ep_calib_fill), in scrambled order (ep_calib_fill_shuffled), torch\'s fill, and the copy '
                          'kernel with its loads taken out (ep_scatter_quant_stores_only)')
     ap.add_argument('--combine-blocks-per-cu', type=int, default=None,
-                    help='tuning: workgroups of a combine kernel a CU holds at once (library default 4; 0: no cap)')
+                    help='tuning: workgroups of a combine kernel a CU holds at once (library default: by top-k; 0: no cap)')
     ap.add_argument('--samples', type=int, default=50, help='isolated, cache-flushed launches per kernel')
     args = ap.parse_args()
     if args.graph:

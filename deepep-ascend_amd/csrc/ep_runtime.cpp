@@ -123,14 +123,26 @@ Kernels g_k;
 bool g_fp8_hw = true;
 bool g_stores_only = false;     // calibration: the fused-quantising copy kernel runs without its loads of x
 // Workgroups of the single-partition combine kernel a CU holds at once, enforced through an unused dynamic LDS
-// allocation (0: no cap, the registers decide: 5 to 7).  Measured at the headline shape (top-6, 12 row fetches of
-// 1 KiB a wave): 7 a CU 291 us, 5: 287, 4: 275-278, 3: 282, 2: 320; top-8 at 4096 tokens and the two-phase
-// kernels of the partitioned path do not react to it.
-int g_combine_blocks_per_cu = 4;
+// allocation (0: no cap, the registers decide: 5 to 8; negative: chosen by top-k, below).  The gather is fastest
+// with about 192 KiB of row fetches in flight a CU (a wave fetches top-k x 2 KiB): more waves queue more fetches
+// than the memory keeps open.  Measured at 16384 tokens x 7168 (microseconds at 2/3/4/5/6 workgroups and uncapped):
+//   top-2  183 145 129 123 120 122      top-4  257 214 196 196 199 203
+//   top-6  322 282 274 288 288 289      top-8  397 359 375 378 379 380
+// and for the kernel that takes any top-k: top-1 best uncapped, top-3 at 6, top-5 at 5, top-7 to top-16 at 4.
+// The two-phase kernels of the partitioned path do not react to it.
+int g_combine_blocks_per_cu = -1;
 constexpr unsigned kLdsBytesPerCu = 160 * 1024;
-unsigned combine_lds_cap() {
-    if (g_combine_blocks_per_cu <= 0) return 0;
-    const unsigned share = kLdsBytesPerCu / (unsigned)g_combine_blocks_per_cu;
+unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks) {
+    int n = g_combine_blocks_per_cu;
+    if (n < 0) {
+        // a launch that fills the machine less than about twice over wants every wave it can get
+        // (1024 tokens, top-6: 23.8 us uncapped, 25.4 at four workgroups; from 4096 tokens on the cap costs nothing)
+        if (num_row_blocks < 4096) n = 0;
+        else if (specialised) n = num_topk <= 2 ? 0 : num_topk <= 4 ? 5 : num_topk <= 6 ? 4 : 3;
+        else n = num_topk <= 2 ? 0 : num_topk == 3 ? 6 : num_topk <= 5 ? 5 : 4;
+    }
+    if (n <= 0) return 0;
+    const unsigned share = kLdsBytesPerCu / (unsigned)n;
     return std::min(64u * 1024u, share - 1024u);       // n of them fit a CU, n + 1 do not
 }
 int g_fold_max_blocks = 256;    // up to this many layout workgroups the slot assignment sums the block counts itself
@@ -1179,7 +1191,7 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
             const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(num_combined_tokens, EP_ROW_THREADS);
             if (grid == 0) return;
-            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, combine_lds_cap(), a.stream, ca);
+            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, combine_lds_cap(K, kidx != 0, ca.num_row_blocks), a.stream, ca);
         } else {
             check_peers(b, [&](const ep_buffer& p) { return p.num_partials >= b->num_partials; },
                         "its owner-side reduce (phase 0) comes before any token-side reduce");

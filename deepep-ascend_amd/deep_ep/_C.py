@@ -256,7 +256,8 @@ def set_calibration_stores_only(enable: bool) -> None:
 
 
 def set_combine_blocks_per_cu(num_blocks: int) -> None:
-    """Tuning: workgroups of a combine kernel a compute unit holds at once (0: no cap).  Results do not depend on it."""
+    """Tuning: workgroups of a combine kernel a compute unit holds at once (0: no cap; negative: chosen by
+    top-k, the default).  Results do not depend on it."""
     _ep_set_combine_cap(int(num_blocks))
 
 
