@@ -962,6 +962,26 @@ __device__ __forceinline__ u32x4 add_biases(const EpCombineArgs& a, int t, int v
     return pack8(acc);
 }
 
+// The same with the bias vectors already in registers (fetched together with the rows): the biases that exist, in
+// order, then the partial.  (Registers of their own and uniform flags: a run-time index into an array of loaded
+// vectors would make the compiler wait for the loads where they are issued.)
+__device__ __forceinline__ u32x4 add_loaded_biases(bool has0, u32x4 x0, bool has1, u32x4 x1, u32x4 partial) {
+    if (!has0 && !has1) return partial;
+    float acc[8], g[8];
+    if (has0) {
+        unpack8(x0, acc);
+        if (has1) {
+            unpack8(x1, g);
+            for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q];
+        }
+    } else {
+        unpack8(x1, acc);
+    }
+    unpack8(partial, g);
+    for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q];
+    return pack8(acc);
+}
+
 // Tokens with no valid slot are never received: their output is the bias sum (or zero).
 __device__ __forceinline__ void combine_unrouted(const EpCombineArgs& a) {
     const int lane = lane_id();
@@ -1075,7 +1095,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     }
 
     u32x4* out = (u32x4*)out_row;
-    const bool has_bias = a.bias_0 != nullptr || a.bias_1 != nullptr;
+    const bool has0 = a.bias_0 != nullptr, has1 = a.bias_1 != nullptr;
     const bool weighted = MODE == EP_COMBINE_FUSED && a.weighted;
     // Owner side with whole rows per task: a received row mostly has a single slot among this partition's few
     // experts, and its partial is then that row verbatim: up to 16 vectors a lane in flight, no arithmetic.
@@ -1103,22 +1123,27 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     // by them has read them; the other tasks hold zeros
     const u32x4 zero = {0u, 0u, 0u, 0u};
     if (KT > 0) {
-        // Every load of the task is issued before the first add: the biases of the token (token-side reduce), then
+        // Every load of the task is issued before the first add: the biases of the token (not on the owner side), then
         // both 16-byte vectors of every input row.  The two vectors are then reduced one after the other, which
         // keeps the live registers at the loaded vectors plus one accumulator (72 VGPRs at K = 6: seven waves a SIMD).
-        u32x4 b0[2], b1[2], d0[KT > 0 ? KT : 1], d1[KT > 0 ? KT : 1];
-        int nb = 0;
-        if (MODE == EP_COMBINE_FINAL) {
-            const void* biases[2] = {a.bias_0, a.bias_1};
-#pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                if (biases[b] == nullptr) continue;
-                const u32x4* bp = (const u32x4*)biases[b] + (int64_t)t * nvec;
-                b0[nb] = live0 ? bp[v0] : zero;
-                b1[nb] = live1 ? bp[v1] : zero;
-                ++nb;
+        u32x4 d0[KT > 0 ? KT : 1], d1[KT > 0 ? KT : 1];
+        // bias vectors: p0* of bias_0, p1* of bias_1, *a for the first vector of the task, *b for the second
+        u32x4 p0a = zero, p0b = zero, p1a = zero, p1b = zero;
+        if (MODE != EP_COMBINE_PARTIAL) {
+            if (has0) {
+                const u32x4* bp = (const u32x4*)a.bias_0 + (int64_t)t * nvec;
+                if (live0) p0a = __builtin_nontemporal_load(bp + v0);
+                if (live1) p0b = __builtin_nontemporal_load(bp + v1);
+            }
+            if (has1) {
+                const u32x4* bp = (const u32x4*)a.bias_1 + (int64_t)t * nvec;
+                if (live0) p1a = __builtin_nontemporal_load(bp + v0);
+                if (live1) p1b = __builtin_nontemporal_load(bp + v1);
             }
         }
+        // token side: the biases open the one accumulation; single partition: they are added to the rounded sum of
+        // the rows in a second one (the two levels of the reference)
+        const bool first0 = MODE == EP_COMBINE_FINAL && has0, first1 = MODE == EP_COMBINE_FINAL && has1;
 #pragma unroll
         for (int j = 0; j < KT; ++j) {
             const int s = readlane(myslot, j);
@@ -1128,13 +1153,18 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
         }
         // inputs in order: b0, b1, then the rows in ascending position; zero inputs -> zeros, one input -> verbatim
         // copy, more -> one rounding of the fp32 sum (a weighted single row is a product: rounded as well)
-        auto reduce = [&](const u32x4* bias, const u32x4* d) -> u32x4 {
+        auto reduce = [&](u32x4 x0, u32x4 x1, const u32x4* d) -> u32x4 {
             float acc[8], g[8];
             u32x4 first = zero;
             int nin = 0;
-            for (int b = 0; b < nb; ++b) {
-                unpack8(bias[b], g);
-                if (nin == 0) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; first = bias[b]; }
+            if (first0) {
+                unpack8(x0, acc);
+                first = x0;
+                ++nin;
+            }
+            if (first1) {
+                unpack8(x1, g);
+                if (nin == 0) { for (int q = 0; q < 8; ++q) acc[q] = g[q]; first = x1; }
                 else { for (int q = 0; q < 8; ++q) acc[q] = acc[q] + g[q]; }
                 ++nin;
             }
@@ -1155,13 +1185,13 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
             return first;
         };
         if (live0) {
-            u32x4 res = reduce(b0, d0);
-            if (MODE == EP_COMBINE_FUSED && has_bias) res = add_biases(a, t, v0, true, res);
+            u32x4 res = reduce(p0a, p1a, d0);
+            if (MODE == EP_COMBINE_FUSED) res = add_loaded_biases(has0, p0a, has1, p1a, res);
             stream_store<EP_COMBINE_ST_POL>(out + v0, res);
         }
         if (live1) {
-            u32x4 res = reduce(b1, d1);
-            if (MODE == EP_COMBINE_FUSED && has_bias) res = add_biases(a, t, v1, true, res);
+            u32x4 res = reduce(p0b, p1b, d1);
+            if (MODE == EP_COMBINE_FUSED) res = add_loaded_biases(has0, p0b, has1, p1b, res);
             stream_store<EP_COMBINE_ST_POL>(out + v1, res);
         }
         continue;
@@ -1169,6 +1199,19 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     float acc0[8], acc1[8];
     u32x4 res0 = zero, res1 = zero;
     int nin = 0;                                              // inputs accumulated so far
+    u32x4 p0a = zero, p0b = zero, p1a = zero, p1b = zero;     // single partition: biases fetched ahead of the rows
+    if (MODE == EP_COMBINE_FUSED) {
+        if (has0) {
+            const u32x4* bp = (const u32x4*)a.bias_0 + (int64_t)t * nvec;
+            if (live0) p0a = __builtin_nontemporal_load(bp + v0);
+            if (live1) p0b = __builtin_nontemporal_load(bp + v1);
+        }
+        if (has1) {
+            const u32x4* bp = (const u32x4*)a.bias_1 + (int64_t)t * nvec;
+            if (live0) p1a = __builtin_nontemporal_load(bp + v0);
+            if (live1) p1b = __builtin_nontemporal_load(bp + v1);
+        }
+    }
     if (MODE == EP_COMBINE_FINAL) {
         const void* biases[2] = {a.bias_0, a.bias_1};
 #pragma unroll
@@ -1176,8 +1219,8 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
             if (biases[b] == nullptr) continue;
             const u32x4* bp = (const u32x4*)biases[b] + (int64_t)t * nvec;
             u32x4 e0 = zero, e1 = zero;
-            if (live0) e0 = bp[v0];
-            if (live1) e1 = bp[v1];
+            if (live0) e0 = __builtin_nontemporal_load(bp + v0);
+            if (live1) e1 = __builtin_nontemporal_load(bp + v1);
             float g0[8], g1[8];
             unpack8(e0, g0);
             unpack8(e1, g1);
@@ -1209,11 +1252,11 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
         res1 = pack8(acc1);
     }
     if (live0) {
-        if (MODE == EP_COMBINE_FUSED && has_bias) res0 = add_biases(a, t, v0, true, res0);
+        if (MODE == EP_COMBINE_FUSED) res0 = add_loaded_biases(has0, p0a, has1, p1a, res0);
         stream_store<EP_COMBINE_ST_POL>(out + v0, res0);
     }
     if (live1) {
-        if (MODE == EP_COMBINE_FUSED && has_bias) res1 = add_biases(a, t, v1, true, res1);
+        if (MODE == EP_COMBINE_FUSED) res1 = add_loaded_biases(has0, p0b, has1, p1b, res1);
         stream_store<EP_COMBINE_ST_POL>(out + v1, res1);
     }
     }

@@ -129,10 +129,11 @@ bool g_stores_only = false;     // calibration: the fused-quantising copy kernel
 //   top-2  183 145 129 123 120 122      top-4  257 214 196 196 199 203
 //   top-6  322 282 274 288 288 289      top-8  397 359 375 378 379 380
 // and for the kernel that takes any top-k: top-1 best uncapped, top-3 at 6, top-5 at 5, top-7 to top-16 at 4.
+// A bias row is one more row a wave fetches: top-6 with one / two biases 358 316 323 332 / 387 349 370 375 at 2/3/4/5.
 // The two-phase kernels of the partitioned path do not react to it.
 int g_combine_blocks_per_cu = -1;
 constexpr unsigned kLdsBytesPerCu = 160 * 1024;
-unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks) {
+unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks) {     // num_topk: rows a wave fetches, biases included
     int n = g_combine_blocks_per_cu;
     if (n < 0) {
         // a launch that fills the machine less than about twice over wants every wave it can get
@@ -1191,7 +1192,7 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
             const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(num_combined_tokens, EP_ROW_THREADS);
             if (grid == 0) return;
-            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, combine_lds_cap(K, kidx != 0, ca.num_row_blocks), a.stream, ca);
+            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, combine_lds_cap(K + (ca.bias_0 != nullptr) + (ca.bias_1 != nullptr), kidx != 0, ca.num_row_blocks), a.stream, ca);
         } else {
             check_peers(b, [&](const ep_buffer& p) { return p.num_partials >= b->num_partials; },
                         "its owner-side reduce (phase 0) comes before any token-side reduce");
