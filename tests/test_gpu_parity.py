@@ -213,6 +213,41 @@ def test_column_major_scales(R, rank, do_cpu_sync):
     buf.destroy()
 
 
+@pytest.mark.parametrize('packs', [3, 4, 66])
+@pytest.mark.parametrize('alignment', [1, 2])
+def test_column_major_two_byte_packs_of_any_shape(packs, alignment):
+    """Pre-quantised input whose scale packs are any 2-byte type, asked for as columns: odd and even pack
+    counts, odd and even row counts (the transposing kernel moves pairs of packs where both are even and
+    single ones otherwise), more columns than one tile holds."""
+    de = _deep_ep()
+    T, H, E, K = 71, 128, 4, 2
+    topk, w = make_routing(T, E, K, seed=3, masked=0.3)
+    g = torch.Generator().manual_seed(packs)
+    xq = torch.randint(0, 255, (T, H), generator=g, dtype=torch.uint8)
+    sf = torch.randint(-32768, 32767, (T, packs), generator=g, dtype=torch.int16)
+    seen = set()
+    for drop in (0, 1):                     # one token less changes the parity of the row count at alignment 1
+        tk = topk.clone()
+        if drop:                            # token 0 gets one selection more or less than it had
+            tk[0] = torch.tensor([0, -1] if int((topk[0] >= 0).sum()) != 1 else [0, 1])
+        lay = O.rank_share_layout(tk.numpy(), E, 1, 0, alignment, T)
+        ex, es, _ = O.rank_share_dispatch(xq.numpy(), sf.numpy().view(np.uint8).reshape(T, -1), w.numpy(), lay)
+        buf = _buffer(T, H, K, fp8=True)
+        (rx, rsf), _, _, handle, _ = buf.dispatch((xq.view(torch.float8_e4m3fn).to(DEV), sf.to(DEV)), topk_idx=tk.to(DEV),
+                                                  topk_weights=w.to(DEV), num_experts=E, num_max_tokens_per_rank=T,
+                                                  expert_alignment=alignment, do_expand=True, do_zero_padding=True,
+                                                  use_tma_aligned_col_major_sf=True)
+        torch.cuda.synchronize()
+        n = lay['num_expanded_tokens']
+        seen.add(n % 2)
+        assert rsf.shape == (n, packs) and rsf.stride() == (1, n)
+        assert np.array_equal(rx.view(torch.uint8).cpu().numpy(), ex)
+        assert np.array_equal(rsf.cpu().numpy(), es.view(np.int16).reshape(n, packs))
+        buf.destroy()
+    if alignment == 1:
+        assert seen == {0, 1}               # both parities of the row count were exercised
+
+
 def test_fp8_hardware_conversion_matches_integer_conversion():
     """Every fp32 bit pattern with |x| <= 464 (the quantiser never exceeds 448*(1+2^-23))."""
     de = _deep_ep()
