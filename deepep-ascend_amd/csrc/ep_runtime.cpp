@@ -133,12 +133,14 @@ bool g_stores_only = false;     // calibration: the fused-quantising copy kernel
 // The two-phase kernels of the partitioned path do not react to it.
 int g_combine_blocks_per_cu = -1;
 constexpr unsigned kLdsBytesPerCu = 160 * 1024;
-unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks) {     // num_topk: rows a wave fetches, biases included
+unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks, int hidden) {     // num_topk: rows a wave fetches, biases included
     int n = g_combine_blocks_per_cu;
     if (n < 0) {
         // a launch that fills the machine less than about twice over wants every wave it can get
-        // (1024 tokens, top-6: 23.8 us uncapped, 25.4 at four workgroups; from 4096 tokens on the cap costs nothing)
-        if (num_row_blocks < 4096) n = 0;
+        // (1024 tokens, top-6: 23.8 us uncapped, 25.4 at four workgroups; from 4096 tokens on the cap costs nothing),
+        // and so do short rows (hidden 512 / 1536, top-8: 113 / 160 us uncapped, 124 / 170 at three; from 2048 on the
+        // cap wins)
+        if (num_row_blocks < 4096 or hidden < 2048) n = 0;
         else if (specialised) n = num_topk <= 2 ? 0 : num_topk <= 4 ? 5 : num_topk <= 6 ? 4 : 3;
         else n = num_topk <= 2 ? 0 : num_topk == 3 ? 6 : num_topk <= 5 ? 5 : 4;
     }
@@ -1192,7 +1194,7 @@ int ep_combine_launch(ep_buffer_t* b, const ep_combine_args_t* pa, int phase) {
             ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
             const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(num_combined_tokens, EP_ROW_THREADS);
             if (grid == 0) return;
-            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, combine_lds_cap(K + (ca.bias_0 != nullptr) + (ca.bias_1 != nullptr), kidx != 0, ca.num_row_blocks), a.stream, ca);
+            launch(g_k.combine[EP_COMBINE_FUSED][kidx], grid, EP_ROW_THREADS, combine_lds_cap(K + (ca.bias_0 != nullptr) + (ca.bias_1 != nullptr), kidx != 0, ca.num_row_blocks, hidden), a.stream, ca);
         } else {
             check_peers(b, [&](const ep_buffer& p) { return p.num_partials >= b->num_partials; },
                         "its owner-side reduce (phase 0) comes before any token-side reduce");
