@@ -1163,30 +1163,52 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
         // Every load of the task is issued before the first add: the biases of the token (not on the owner side), then
         // both 16-byte vectors of every input row.  The two vectors are then reduced one after the other, which
         // keeps the live registers at the loaded vectors plus one accumulator (72 VGPRs at K = 6: seven waves a SIMD).
+        // No load depends on the lane being live: a lane past the end of the row fetches the row's last vector and
+        // stores nothing.  (A load under a per-lane condition has to be merged with the register's old value when it
+        // returns, and the compiler then waits for the first such load before it issues the next.)
+        const int c0 = min(v0, nvec - 1), c1 = min(v1, nvec - 1);
         u32x4 d0[KT > 0 ? KT : 1], d1[KT > 0 ? KT : 1];
         // bias vectors: p0* of bias_0, p1* of bias_1, *a for the first vector of the task, *b for the second
         u32x4 p0a = zero, p0b = zero, p1a = zero, p1b = zero;
         if (MODE != EP_COMBINE_PARTIAL) {
             if (has0) {
                 const u32x4* bp = (const u32x4*)a.bias_0 + (int64_t)t * nvec;
-                if (live0) p0a = __builtin_nontemporal_load(bp + v0);
-                if (live1) p0b = __builtin_nontemporal_load(bp + v1);
+                p0a = __builtin_nontemporal_load(bp + c0);
+                p0b = __builtin_nontemporal_load(bp + c1);
             }
             if (has1) {
                 const u32x4* bp = (const u32x4*)a.bias_1 + (int64_t)t * nvec;
-                if (live0) p1a = __builtin_nontemporal_load(bp + v0);
-                if (live1) p1b = __builtin_nontemporal_load(bp + v1);
+                p1a = __builtin_nontemporal_load(bp + c0);
+                p1b = __builtin_nontemporal_load(bp + c1);
             }
         }
         // token side: the biases open the one accumulation; single partition: they are added to the rounded sum of
         // the rows in a second one (the two levels of the reference)
         const bool first0 = MODE == EP_COMBINE_FINAL && has0, first1 = MODE == EP_COMBINE_FINAL && has1;
+        if (MODE == EP_COMBINE_PARTIAL) {
+            // owner side: a received row has one or two of its K positions on this partition: fetch those only
 #pragma unroll
-        for (int j = 0; j < KT; ++j) {
-            const int s = readlane(myslot, j);
-            if (s < 0) continue;
-            if (live0) d0[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + v0);
-            if (live1) d1[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + v1);
+            for (int j = 0; j < KT; ++j) {
+                const int s = readlane(myslot, j);
+                if (s < 0) continue;
+                d0[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + c0);
+                d1[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + c1);
+            }
+        } else if (nvalid > 0) {
+            // nearly every position is valid: one straight run of 2 K loads with no branch in it, a position without
+            // a row re-reads the first valid one (the same cache lines again) and is left out of the sum below
+            const int s_any = readlane(myslot, (int)__builtin_ctzll(__ballot(myslot >= 0)));
+#pragma unroll
+            for (int j = 0; j < KT; ++j) {
+                const int s = readlane(myslot, j);
+                const int64_t row = (int64_t)(s >= 0 ? s : s_any) * yvec;
+                d0[j] = __builtin_nontemporal_load(y + row + c0);
+                d1[j] = __builtin_nontemporal_load(y + row + c1);
+                // sixteen and more fetches a wave are better sent in two goes, the first row ahead of the others
+                // (top-8 at 16384 / 32768 tokens: 354 / 707 us against 362 / 730 all at once; top-6 and below lose:
+                // 277 against 272)
+                if (KT >= 8 && j == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
         }
         // inputs in order: b0, b1, then the rows in ascending position; zero inputs -> zeros, one input -> verbatim
         // copy, more -> one rounding of the fp32 sum (a weighted single row is a product: rounded as well)

@@ -124,12 +124,12 @@ bool g_fp8_hw = true;
 bool g_stores_only = false;     // calibration: the fused-quantising copy kernel runs without its loads of x
 // Workgroups of the single-partition combine kernel a CU holds at once, enforced through an unused dynamic LDS
 // allocation (0: no cap, the registers decide: 5 to 8; negative: chosen by top-k, below).  The gather is fastest
-// with about 192 KiB of row fetches in flight a CU (a wave fetches top-k x 2 KiB): more waves queue more fetches
-// than the memory keeps open.  Measured at 16384 tokens x 7168 (microseconds at 2/3/4/5/6 workgroups and uncapped):
-//   top-2  183 145 129 123 120 122      top-4  257 214 196 196 199 203
-//   top-6  322 282 274 288 288 289      top-8  397 359 375 378 379 380
+// with about 150 KiB of row fetches in flight a CU (a wave fetches top-k x 2 KiB): more waves queue more fetches
+// than the memory keeps open.  Measured at 16384 tokens x 7168 (microseconds at 2/3/4/5 workgroups and uncapped):
+//   top-2  175 140 126 120 120      top-4  233 201 194 199 200
+//   top-6  297 272 286 289 291      top-8  385 354 377 378 376
 // and for the kernel that takes any top-k: top-1 best uncapped, top-3 at 6, top-5 at 5, top-7 to top-16 at 4.
-// A bias row is one more row a wave fetches: top-6 with one / two biases 358 316 323 332 / 387 349 370 375 at 2/3/4/5.
+// A bias row is one more row a wave fetches: top-6 with one / two biases 326 311 329 336 / 358 350 373 377 at 2/3/4/5.
 // The two-phase kernels of the partitioned path do not react to it.
 int g_combine_blocks_per_cu = -1;
 constexpr unsigned kLdsBytesPerCu = 160 * 1024;
@@ -141,7 +141,7 @@ unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks, int
         // and so do short rows (hidden 512 / 1536, top-8: 113 / 160 us uncapped, 124 / 170 at three; from 2048 on the
         // cap wins)
         if (num_row_blocks < 4096 or hidden < 2048) n = 0;
-        else if (specialised) n = num_topk <= 2 ? 0 : num_topk <= 4 ? 5 : num_topk <= 6 ? 4 : 3;
+        else if (specialised) n = num_topk <= 2 ? 0 : num_topk <= 4 ? 4 : 3;
         else n = num_topk <= 2 ? 0 : num_topk == 3 ? 6 : num_topk <= 5 ? 5 : 4;
     }
     if (n <= 0) return 0;

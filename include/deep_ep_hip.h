@@ -177,8 +177,8 @@ int64_t ep_dispatch_stamp(ep_buffer_t* buf);
 void ep_set_layout_fold_max_blocks(int num_blocks);
 
 /* Tuning: workgroups (of 4 waves) of the single-partition combine kernel that a compute unit holds at once;
- * 0 lifts the cap, a negative value lets the library choose by top-k (the default: 3 at top-8, 4 at top-6,
- * 5 at top-4, none at top-2 and for launches too small to fill the machine twice).  Results do not depend on it. */
+ * 0 lifts the cap, a negative value lets the library choose by top-k (the default: 3 at top-6 and top-8,
+ * 4 at top-4, none at top-2 and for launches too small to fill the machine twice).  Results do not depend on it. */
 void ep_set_combine_blocks_per_cu(int num_blocks);
 
 /* More than one partition, non-cached dispatch: the receive side of launch_dispatch and the slot
