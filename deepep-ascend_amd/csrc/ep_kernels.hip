@@ -624,6 +624,7 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
     const int lane = lane_id();
     const int K = a.num_topk;
     int myslot = -1, t;
+    float early_w = 0.0f;          // gate weight fetched ahead of its use (token-walking expand)
     if (PACK) {
         uint64_t mybase = 0;
         t = i;
@@ -674,10 +675,16 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
         // the receive stream a token became is only needed for its metadata row
         t = i;
         if (lane < K) myslot = a.slot_map[(int64_t)t * K + lane];
+        // the task that writes the token's metadata row and weights fetches what it needs for that in the same trip
+        // (both are indexed by the token alone; tok_row holds nothing meaningful for a token nobody receives)
+        int row = -1;
+        if (part == 0) {
+            row = a.tok_row[t];
+            if (a.recv_topk_weights != nullptr && lane < K) early_w = a.topk_weights[(int64_t)t * K + lane];
+        }
         const uint64_t vm = __ballot(myslot >= 0);
         if (vm == 0) return false;                       // a token nobody receives
         if (part == 0) {
-            const int row = a.tok_row[t];
             const int master = 63 - __builtin_clzll(vm);
             // [slot_0 .. slot_{K-1}, src_token_global_idx, last local j]  (dispatch_copy_epilogue.hpp:514-522)
             const int v = lane < K ? myslot : (lane == K ? a.rank_idx * a.max_tokens + t : master);
@@ -693,7 +700,7 @@ __device__ __forceinline__ bool scatter_row_prologue(const EpScatterArgs& a, int
     if (lane < K && (myslot < 0 || myslot >= a.num_out_rows)) myslot = -1;
     c.src_row = (int64_t)t;
     if (part == 0 && a.recv_topk_weights != nullptr && lane < K && myslot >= 0)
-        a.recv_topk_weights[myslot] = a.topk_weights[(int64_t)t * K + lane];
+        a.recv_topk_weights[myslot] = a.cached ? a.topk_weights[(int64_t)t * K + lane] : early_w;
     c.t = t;
     c.myslot = myslot;
     return true;
@@ -1100,6 +1107,9 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
         if (MODE == EP_COMBINE_PARTIAL && (group < 0 || group >= a.num_groups)) return;
     }
     const int nvalid = __popcll(__ballot(myslot >= 0));
+    // Owner side with whole rows per task: a received row mostly has a single slot among this partition's few
+    // experts, and its partial is then that row verbatim: up to 16 vectors a lane in flight, no arithmetic.
+    const bool verbatim = MODE == EP_COMBINE_PARTIAL && a.whole_rows && nvalid == 1;
     const int nvec = a.hidden >> 3;
     const int64_t yvec = a.y_row_bytes >> 4;
     const u32x4* y = (const u32x4*)a.y;
@@ -1113,10 +1123,26 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     if (MODE == EP_COMBINE_FINAL) {
         if (part == 0 && a.combined_topk_weights != nullptr) {
             unsigned acc = 0;
-            for (int j = 0; j < K; ++j) {
-                const int s = readlane(myslot, j);
-                if (s < 0) continue;
-                if (lane < K) acc |= ((const unsigned*)((const char*)a.y + (int64_t)s * a.y_row_bytes + (a.hidden << 1)))[lane];
+            if (KT > 0 && nvalid > 0) {
+                // the weight vectors of all masters in one trip: no branch and no per-lane condition between the
+                // loads (a position that is no master re-reads the first master's vector and is left out)
+                const int s_any = readlane(myslot, (int)__builtin_ctzll(__ballot(myslot >= 0)));
+                const int wl = min(lane, K - 1);
+                unsigned wv[KT > 0 ? KT : 1];
+#pragma unroll
+                for (int j = 0; j < KT; ++j) {
+                    const int s = readlane(myslot, j);
+                    wv[j] = ((const unsigned*)((const char*)a.y + (int64_t)(s >= 0 ? s : s_any) * a.y_row_bytes + (a.hidden << 1)))[wl];
+                }
+#pragma unroll
+                for (int j = 0; j < KT; ++j)
+                    if (readlane(myslot, j) >= 0) acc |= wv[j];
+            } else {
+                for (int j = 0; j < K; ++j) {
+                    const int s = readlane(myslot, j);
+                    if (s < 0) continue;
+                    if (lane < K) acc |= ((const unsigned*)((const char*)a.y + (int64_t)s * a.y_row_bytes + (a.hidden << 1)))[lane];
+                }
             }
             if (lane < K) ((unsigned*)a.combined_topk_weights)[(int64_t)t * K + lane] = acc;
         }
@@ -1126,7 +1152,8 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
         if (part == 0 && lane < K) {
             if (MODE == EP_COMBINE_FUSED && a.combined_topk_weights != nullptr)
                 a.combined_topk_weights[(int64_t)t * K + lane] = myw;
-            if (MODE == EP_COMBINE_PARTIAL && a.expanded_weights != nullptr)
+            // (the verbatim path below stores them behind its row fetches, so that the two trips become one)
+            if (MODE == EP_COMBINE_PARTIAL && a.expanded_weights != nullptr && !verbatim)
                 ((float*)(out_row + (a.hidden << 1)))[lane] = myw;
         }
     }
@@ -1134,9 +1161,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     u32x4* out = (u32x4*)out_row;
     const bool has0 = a.bias_0 != nullptr, has1 = a.bias_1 != nullptr;
     const bool weighted = MODE == EP_COMBINE_FUSED && a.weighted;
-    // Owner side with whole rows per task: a received row mostly has a single slot among this partition's few
-    // experts, and its partial is then that row verbatim: up to 16 vectors a lane in flight, no arithmetic.
-    if (MODE == EP_COMBINE_PARTIAL && a.whole_rows && nvalid == 1) {
+    if (verbatim) {
         const int s1 = readlane(myslot, __builtin_ctzll(__ballot(myslot >= 0)));
         const u32x4* src = y + (int64_t)s1 * yvec;
         for (int vb = lane; vb < nvec; vb += 16 * WAVE) {
@@ -1144,6 +1169,7 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
 #pragma unroll
             for (int u = 0; u < 16; ++u)
                 if (vb + u * WAVE < nvec) d[u] = __builtin_nontemporal_load(src + vb + u * WAVE);
+            if (vb == lane && lane < K && a.expanded_weights != nullptr) ((float*)(out_row + (a.hidden << 1)))[lane] = myw;
 #pragma unroll
             for (int u = 0; u < 16; ++u)
                 if (vb + u * WAVE < nvec) stream_store<EP_COMBINE_ST_POL>(out + vb + u * WAVE, d[u]);
