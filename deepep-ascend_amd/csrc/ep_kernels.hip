@@ -148,14 +148,25 @@ __device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s
     }
     const int64_t base = (int64_t)blockIdx.x * n;
     const int64_t total = (int64_t)a.num_tokens * K;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        int e = -1;
-        if (base + i < total) {
-            const int64_t v = a.topk_idx[base + i];
-            e = (v >= 0 && v < a.num_experts) ? (int)v : -1;
+    if (total <= 0) {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) s_key[i] = s_rk[i] = -1;
+        return;
+    }
+    // four loads a thread in flight, none under a per-lane condition (an entry past the end re-reads the last one
+    // and is masked): the ids come from memory, and one trip for a workgroup's entries is all this pass waits for
+    for (int i0 = threadIdx.x; i0 < n; i0 += 4 * blockDim.x) {
+        int64_t v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = a.topk_idx[min(base + i0 + u * (int)blockDim.x, total - 1)];
+        __builtin_amdgcn_sched_barrier(0);      // (the scheduler otherwise uses the first value before it issues the other loads)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = i0 + u * (int)blockDim.x;
+            if (i >= n) break;
+            const int e = (base + i < total && v[u] >= 0 && v[u] < a.num_experts) ? (int)v[u] : -1;
+            s_key[i] = (short)e;
+            s_rk[i] = (short)(e < 0 ? -1 : e / a.experts_per_rank);
         }
-        s_key[i] = (short)e;
-        s_rk[i] = (short)(e < 0 ? -1 : e / a.experts_per_rank);
     }
 }
 
