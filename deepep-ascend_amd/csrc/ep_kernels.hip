@@ -315,7 +315,19 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             pre[k] = a.blk_cnt[(int64_t)b * a.cnt_stride + c];
             tot[k] = a.col_total[c];
         }
-    } else if (a.scan_mode == EP_LAYOUT_FOLDED) {
+    }
+    // This workgroup's expert ids are asked for before the sums below and land while those wait for their rows
+    // (send side, up to four ids a thread).
+    const int nkeys = EP_TOKENS_PER_BLOCK * K;
+    const int64_t key_base = (int64_t)b * nkeys, key_total = (int64_t)a.num_tokens * K;
+    const bool keys_early = a.scan_mode == EP_LAYOUT_FOLDED && !a.recv_mode && nkeys <= 4 * EP_LAYOUT_THREADS && key_total > 0;
+    int64_t pk[4] = {-1, -1, -1, -1};
+    if (keys_early) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) pk[u] = a.topk_idx[min(key_base + tid + u * EP_LAYOUT_THREADS, key_total - 1)];
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (a.scan_mode == EP_LAYOUT_FOLDED) {
         // ep_layout_count has finished and left plain counts: sum the rows before this workgroup's (and all
         // rows) here.  A thread takes 4 adjacent columns (one 16-byte load a row) of every S-th row, EP_FOLD_DEPTH
         // loads in flight (the rows come from memory: other XCDs wrote them); the S partial sums of a column
@@ -368,7 +380,18 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
 
     // ---- A: stage this block's keys, clear the per-wave counters ----
     for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
-    layout_load_keys(a, s_key, s_rk, s_psum, num_rows);
+    if (keys_early) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = tid + u * EP_LAYOUT_THREADS;
+            if (i >= nkeys) break;
+            const int e = (key_base + i < key_total && pk[u] >= 0 && pk[u] < a.num_experts) ? (int)pk[u] : -1;
+            s_key[i] = (short)e;
+            s_rk[i] = (short)(e < 0 ? -1 : e / a.experts_per_rank);
+        }
+    } else {
+        layout_load_keys(a, s_key, s_rk, s_psum, num_rows);
+    }
     __syncthreads();
 
     // ---- B: per-wave counts: wave w owns entries [w*epw, (w+1)*epw) of this block's chunk ----
