@@ -491,7 +491,7 @@ class EPBuffer(BufferBase):
                 c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
                 c_list = (ctypes.c_int * max(1, num_local_experts))()
                 _check(_ep_wait(self._h, ctypes.byref(c_recv), ctypes.byref(c_exp), c_list))
-                return c_recv.value, c_exp.value, [c_list[i] for i in range(num_local_experts)]
+                return c_recv.value, c_exp.value, c_list[:num_local_experts]       # (a slice of a ctypes array is a list)
 
             if cached_mode:
                 num_recv, num_expanded = cached_num_recv_tokens, cached_num_expanded_tokens
