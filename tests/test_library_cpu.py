@@ -195,3 +195,14 @@ def test_committed_traffic_summary_belongs_to_the_kernel_sources():
     # measured traffic = algorithmic bytes (+ the zero padding the copy kernel also writes), nothing re-read
     assert 1.0 <= traffic['ep_scatter_quant'] / (964427776 + 115495936) < 1.02
     assert 1.0 <= traffic['ep_combine_k6'] / 1646264320 < 1.02
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU's share is all this path has: asked for more, bench.py says so and exits with a usage error."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2
+    assert 'one GPU' in r.stderr and r.stdout.strip() == ''
