@@ -167,11 +167,39 @@ def cpu_baseline(H, E, K, A, fp8, sample_tokens, budget_s=12.0, max_passes=16):
             'small_case': cpu_small_case()}
 
 
-def calibrate_write(deep_ep, timed, n, dispatch, handle, T, H, K, n_valid, n_recv, pad_bytes, dev, us_scatter):
-    """Pure writes of the byte count the fused FP8 copy kernel writes (payload, scales, weights, metadata, zero
-    padding), same sampling as the kernels: 4 KiB chunks in address order, in scrambled order, torch's fill,
-    and the copy kernel itself with its loads of x taken out (same stores to the same slots)."""
-    wbytes = n_valid * (H + (H // 128) * 4 + 4) + n_recv * (K + 2) * 4 + pad_bytes
+def calib_scatter_args(ep_calib, xg, wg, handle, recv_x, recv_sf, recv_w, T, H, K, E, A):
+    """The fused dispatch of this run as the calibration library's kernels take it (plain pointers; the tensors
+    are returned as well so that they outlive the launches)."""
+    a = ep_calib.ScatterArgs()
+    num_recv = handle.psum_num_recv_tokens_per_rank[-1:]
+    keep = (xg, wg, handle.recv_src_metadata, num_recv, handle.psum_num_recv_tokens_per_expert, recv_x, recv_sf, recv_w)
+    a.x, a.topk_weights = xg.data_ptr(), wg.data_ptr()
+    a.recv_src_metadata, a.num_recv = handle.recv_src_metadata.data_ptr(), num_recv.data_ptr()
+    a.psum_expert = handle.psum_num_recv_tokens_per_expert.data_ptr()
+    a.recv_x, a.recv_sf, a.recv_topk_weights = recv_x.data_ptr(), recv_sf.data_ptr(), recv_w.data_ptr()
+    a.num_tokens, a.hidden, a.num_topk, a.num_experts, a.expert_alignment = T, H, K, E, A
+    a.num_recv_rows, a.num_out_rows, a.do_zero_padding = handle.recv_src_metadata.size(0), recv_x.size(0), 1
+    return a, keep
+
+
+def dispatch_ceiling(ep_calib, timed, n, cargs, us_scatter):
+    """What bounds the token-major copy kernel, from two kernels of the calibration code object run here: its
+    store stream alone (the same tasks storing to the same slots, nothing read but the slots) and its loads
+    of x alone.  On this memory system reads and writes share the time: the sum is the kernel's floor."""
+    med = lambda v: v[len(v) // 2]  # noqa: E731
+    st = med(timed(lambda: ep_calib.scatter('stores_only', cargs), n))
+    rd = med(timed(lambda: ep_calib.scatter('read_rows', cargs), n))
+    return {'stores_only_us': round(st, 2), 'read_us': round(rd, 2), 'sum_us': round(st + rd, 2),
+            'copy_kernel_us': round(us_scatter, 2), 'copy_kernel_over_sum': round(us_scatter / (st + rd), 3),
+            'kernels': 'ep_calib_scatter_stores_only, ep_calib_read_rows (ep_calib.hsaco), isolated flushed medians'}
+
+
+def calibrate_write(ep_calib, timed, n, cargs, T, H, K, n_valid, n_recv, pad_bytes, dev, us_scatter, meta):
+    """Pure writes of the byte count the fused FP8 copy kernel writes (payload, scales, weights, zero padding),
+    same sampling as the kernels: 4 KiB chunks in address order, in scrambled order, 256 write fronts in lock
+    step, a mixed read/write stream in address order, torch's fill; then the formulations of the copy kernel
+    that write in destination order (one pass, and quantise-then-copy), whole and taken apart."""
+    wbytes = n_valid * (H + (H // 128) * 4 + 4) + pad_bytes
     seq_bytes = -(-wbytes // 4096) * 4096
     pow2_bytes = 4096 << (seq_bytes // 4096 - 1).bit_length()          # the scrambled order needs 2^k chunks
     area = torch.empty(pow2_bytes, dtype=torch.uint8, device=dev)
@@ -181,21 +209,59 @@ def calibrate_write(deep_ep, timed, n, dispatch, handle, T, H, K, n_valid, n_rec
     def entry(name, us, nbytes, note):
         res[name] = {'us': round(us, 2), 'bytes': nbytes, 'gbs': round(nbytes / us / 1e3, 1), 'what': note}
 
-    entry('ep_calib_fill', med(timed(lambda: deep_ep._C.calibrate_fill(area[:seq_bytes]), n)), seq_bytes,
+    entry('ep_calib_fill', med(timed(lambda: ep_calib.fill(area[:seq_bytes]), n)), seq_bytes,
           '4 KiB per workgroup, one 16-byte non-temporal store per thread, address order')
-    entry('ep_calib_fill_shuffled', med(timed(lambda: deep_ep._C.calibrate_fill(area, shuffled=1), n)), pow2_bytes,
+    entry('ep_calib_fill_shuffled', med(timed(lambda: ep_calib.fill(area, shuffled=1), n)), pow2_bytes,
           'the same chunks in a scrambled order')
     for unit in (4, 16, 256):                                         # 16 KiB, 64 KiB, 1 MiB
-        entry(f'ep_calib_fill_shuffled_{unit * 4}KiB', med(timed(lambda: deep_ep._C.calibrate_fill(area, shuffled=unit), n)),
+        entry(f'ep_calib_fill_shuffled_{unit * 4}KiB', med(timed(lambda: ep_calib.fill(area, shuffled=unit), n)),
               pow2_bytes, f'runs of {unit} chunks ({unit * 4} KiB) kept together, the runs scrambled')
+    rows = min(448, area.numel() // (256 * H))
+    entry('ep_calib_fronts_256', med(timed(lambda: ep_calib.fronts(area, 256, rows, H, rows * H), n)), 256 * rows * H,
+          f'256 regions filling up in lock step, one {H}-byte row per workgroup (what a gather-formulated dispatch writes)')
+    src = torch.zeros(-(-seq_bytes * 2 // 7 // 4096) * 4096 + 4096, dtype=torch.uint8, device=dev)
+    us = med(timed(lambda: ep_calib.mixed(src, area[:seq_bytes], 2, 7), n))
+    res['ep_calib_mixed_2r7w'] = {'us': round(us, 2), 'bytes_written': seq_bytes, 'bytes_read': seq_bytes * 2 // 7,
+                                  'gbs': round(seq_bytes * 9 / 7 / us / 1e3, 1),
+                                  'what': 'address-ordered 4 KiB chunks, 2 read per 7 written (the copy kernel\'s ratio): '
+                                          'the friendliest stream with the kernel\'s traffic'}
     entry('torch_fill', med(timed(lambda: area[:seq_bytes].zero_(), n)), seq_bytes, 'torch zero_() of the same bytes')
-    deep_ep._C.set_calibration_stores_only(True)
-    try:
-        us = med(timed(lambda: dispatch(handle), n))
-    finally:
-        deep_ep._C.set_calibration_stores_only(False)
-    entry('ep_scatter_quant_stores_only', us, wbytes, 'the copy kernel without its loads of x: same tasks, same stores')
+    del src, area
+
+    def variant(name, what, prep=None):
+        us = med(timed(lambda: ep_calib.scatter(name, cargs), n))
+        res['ep_calib_' + name if not prep else prep] = {'us': round(us, 2), 'what': what}
+
+    variant('token_major', 'the product copy kernel body built into the calibration code object (cached-replay form)')
+    variant('stores_only', 'the copy kernel without its loads of x: same tasks, same stores')
+    variant('read_rows', 'the copy kernel\'s loads of x alone')
     res['ep_scatter_quant'] = {'us': round(us_scatter, 2), 'what': 'the copy kernel (reads x, writes the same bytes)'}
+    # destination order: tasks sorted by slot inside chunks of tokens (a chunk of C tokens leaves one run of about
+    # C * K / E rows in every expert's region)
+    q_rows = torch.empty((T, H), dtype=torch.uint8, device=dev)
+    q_sf = torch.empty((T, H // 128), dtype=torch.float32, device=dev)
+    cargs.q_rows, cargs.q_sf = q_rows.data_ptr(), q_sf.data_ptr()
+    variant('quant_rows', 'two passes, pass 1: every row quantised once, token order, into staging rows')
+    for C in (512, 2048, T):
+        flat, _, _ = ep_calib.build_order(meta, K, C, steered=False)
+        cargs.order, cargs.num_entries, cargs.entries_per_list, cargs.num_lists = flat.data_ptr(), flat.size(0), 0, 0
+        tag = f'chunk{C}'
+        variant('ordered_flat', f'one task per destination row, destination order inside chunks of {C} tokens',
+                f'ep_calib_ordered_flat_{tag}')
+        variant('ordered_flat_stores_only', 'the same without the loads of x', f'ep_calib_ordered_flat_stores_only_{tag}')
+        variant('copy_ordered_flat', 'two passes, pass 2: staged FP8 rows copied in that order', f'ep_calib_copy_ordered_flat_{tag}')
+        if C < T:
+            st, per_list, num_lists = ep_calib.build_order(meta, K, C, steered=True)
+            cargs.order, cargs.num_entries = st.data_ptr(), st.size(0)
+            cargs.entries_per_list, cargs.num_lists = per_list, num_lists
+            variant('ordered_steered', 'the same with all readers of a token on one XCD (x is fetched from memory once)',
+                    f'ep_calib_ordered_steered_{tag}')
+            variant('ordered_steered_stores_only', 'without the loads', f'ep_calib_ordered_steered_stores_only_{tag}')
+            variant('ordered_steered_loads_only', 'without the stores (no zero padding either)',
+                    f'ep_calib_ordered_steered_loads_only_{tag}')
+            variant('copy_ordered_steered', 'two passes, pass 2, steered', f'ep_calib_copy_ordered_steered_{tag}')
+            del st
+        del flat
     return res
 
 
@@ -379,9 +445,9 @@ def main():
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run a plain 1 GiB device copy (known traffic) to scale rocprof byte counters')
     ap.add_argument('--calibrate-write', action='store_true',
-                    help='also time pure writes of the copy kernel\'s byte count: 4 KiB chunks in address order '
-                         '(ep_calib_fill), in scrambled order (ep_calib_fill_shuffled), torch\'s fill, and the copy '
-                         'kernel with its loads taken out (ep_scatter_quant_stores_only)')
+                    help='also time the kernels of the calibration library: pure writes of the copy kernel\'s byte '
+                         'count in several orders, a mixed read/write stream, and the destination-ordered and '
+                         'two-pass formulations of the copy kernel')
     ap.add_argument('--combine-blocks-per-cu', type=int, default=None,
                     help='tuning: workgroups of a combine kernel a CU holds at once (library default: by top-k; 0: no cap)')
     ap.add_argument('--samples', type=int, default=50, help='isolated, cache-flushed launches per kernel')
@@ -617,9 +683,17 @@ def main():
             'scatter_gbs_incl_padding': round((b_d + pad_bytes) / us_scatter / 1e3, 1),
         },
     }
-    if args.calibrate_write and fused:
-        out['write_calibration'] = calibrate_write(deep_ep, timed, n_k, dispatch, handle, T, H, K, n_valid, n_recv,
-                                                   pad_bytes, dev, us_scatter)
+    if fused:
+        # the ceiling of the copy kernel's formulation, from calibration kernels run here (outputs of the first
+        # dispatch serve as their scratch outputs)
+        import ep_calib
+        ep_calib.init()
+        cargs, keep = calib_scatter_args(ep_calib, xg, wg, handle, recv[0], recv[1], recv_w, T, H, K, E, A)
+        roofline['dispatch_ceiling'] = dispatch_ceiling(ep_calib, timed, n_k, cargs, us_scatter)
+        if args.calibrate_write:
+            out['write_calibration'] = calibrate_write(ep_calib, timed, n_k, cargs, T, H, K, n_valid, n_recv, pad_bytes,
+                                                       dev, us_scatter, handle.recv_src_metadata)
+        del keep
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(H, E, K, A, fp8, min(args.cpu_sample_tokens, T))
     buf.destroy()

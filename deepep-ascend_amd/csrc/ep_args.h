@@ -182,12 +182,3 @@ struct EpFp8TestArgs {
     float limit;                  // only |x| <= limit is compared (NaN patterns are skipped)
     int pad;
 };
-
-// Calibration fill: num_chunks chunks of 4 KiB starting at dst.
-struct EpCalibArgs {
-    void* dst;
-    unsigned num_chunks;
-    unsigned value;
-    unsigned unit_chunks;         // scrambled order: consecutive chunks that stay together (a power of two)
-    unsigned pad;
-};

@@ -13,7 +13,8 @@
 //   ep_combine_k<K> / ep_combine_generic                   K-way gather + fp32 reduce back to token order
 //   ep_combine_partial_* / ep_combine_final_*              the same reduce in its owner-side and token-side halves
 //   ep_fp8_selftest                                        hardware vs integer e4m3fn conversion
-//   ep_calib_fill / ep_calib_fill_shuffled / ep_scatter_quant_stores_only   write-path calibration for benchmarks
+// (The calibration code object of the benchmarks, ep_calib.hip, includes this file and instantiates some of
+// its bodies once more; nothing of it is built into this code object.)
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -853,6 +854,8 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_copy_pac
     scatter_copy_body<true>(a);
 }
 
+// (LOADS = false exists for the benchmarks' calibration code object only: the same tasks and stores with a
+// made-up payload in place of the row of x.)
 template <bool HW, bool PACK, bool LOADS = true>
 __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
     if ((int)blockIdx.x >= a.num_row_blocks) {
@@ -900,12 +903,6 @@ __device__ __forceinline__ void scatter_quant_body(const EpScatterArgs& a) {
 
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant(EpScatterArgs a) {
     scatter_quant_body<true, false>(a);
-}
-// Calibration: ep_scatter_quant with the loads of x taken out: the same tasks, the same stores to the same
-// slots (payload, scales, weights, metadata, zero padding), nothing read but the slot map.  Prices the
-// store pattern of the kernel by itself.
-extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_stores_only(EpScatterArgs a) {
-    scatter_quant_body<true, false, false>(a);
 }
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_sw(EpScatterArgs a) {
     scatter_quant_body<false, false>(a);
@@ -1391,27 +1388,6 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
 EP_COMBINE_KERNELS(, EP_COMBINE_FUSED)
 EP_COMBINE_KERNELS(_partial, EP_COMBINE_PARTIAL)
 EP_COMBINE_KERNELS(_final, EP_COMBINE_FINAL)
-
-// ------------------------------------------------------------------------------------------------
-// Calibration writes: what the memory system does with the simplest store patterns.  Workgroup b writes
-// one 4 KiB chunk with one 16-byte non-temporal store per thread; the chunks are visited in address order
-// (ep_calib_fill) or in a scrambled order (ep_calib_fill_shuffled: runs of unit_chunks chunks stay together,
-// run = odd multiplier * index modulo the number of runs, a power of two).
-// ------------------------------------------------------------------------------------------------
-extern "C" __global__ __launch_bounds__(256) void ep_calib_fill(EpCalibArgs a) {
-    u32x4* p = (u32x4*)a.dst + (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const u32x4 v = {a.value, a.value, a.value, a.value};
-    __builtin_nontemporal_store(v, p);
-}
-extern "C" __global__ __launch_bounds__(256) void ep_calib_fill_shuffled(EpCalibArgs a) {
-    // units of unit_chunks consecutive chunks keep their inner order; the units are scrambled
-    const unsigned unit = blockIdx.x / a.unit_chunks, in_unit = blockIdx.x - unit * a.unit_chunks;
-    const unsigned num_units = a.num_chunks / a.unit_chunks;
-    const unsigned chunk = ((unit * 0x9E3779B1u) & (num_units - 1u)) * a.unit_chunks + in_unit;
-    u32x4* p = (u32x4*)a.dst + (int64_t)chunk * 256 + threadIdx.x;
-    const u32x4 v = {a.value, a.value, a.value, a.value};
-    __builtin_nontemporal_store(v, p);
-}
 
 // ------------------------------------------------------------------------------------------------
 // Self-test: hardware e4m3fn conversion against the integer conversion over a range of fp32 bit

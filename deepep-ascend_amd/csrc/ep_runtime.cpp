@@ -114,14 +114,13 @@ struct Kernels {
     hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw, sf_transpose;
     hipFunction_t scatter_copy_pack, scatter_quant_pack, scatter_quant_sw_pack;
     hipFunction_t combine[3][5];     // [mode][generic, k2, k4, k6, k8]
-    hipFunction_t fp8_selftest, scatter_quant_stores_only, calib_fill, calib_fill_shuffled;
+    hipFunction_t fp8_selftest;
     int device = -1;
 };
 
 std::mutex g_mutex;
 Kernels g_k;
 bool g_fp8_hw = true;
-bool g_stores_only = false;     // calibration: the fused-quantising copy kernel runs without its loads of x
 // Workgroups of the single-partition combine kernel a CU holds at once, enforced through an unused dynamic LDS
 // allocation (0: no cap, the registers decide: 5 to 8; negative: chosen by top-k, below).  The gather is fastest
 // with about 150 KiB of row fetches in flight a CU (a wave fetches top-k x 2 KiB): more waves queue more fetches
@@ -188,9 +187,6 @@ void load_kernels(const char* dir) {
         for (int k = 0; k < 5; ++k)
             get(g_k.combine[mode][k], (std::string("ep_combine") + modes[mode] + ks[k]).c_str());
     get(g_k.fp8_selftest, "ep_fp8_selftest");
-    get(g_k.scatter_quant_stores_only, "ep_scatter_quant_stores_only");
-    get(g_k.calib_fill, "ep_calib_fill");
-    get(g_k.calib_fill_shuffled, "ep_calib_fill_shuffled");
     g_k.module = m;
 }
 
@@ -379,22 +375,6 @@ void ep_host_f32_to_e4m3fn(const float* src, uint8_t* dst, int64_t n) {
 }
 
 void ep_set_fp8_hw_convert(int enable) { g_fp8_hw = enable != 0; }
-
-void ep_set_calibration_stores_only(int enable) { g_stores_only = enable != 0; }
-
-int ep_calibrate_fill(void* dst, int64_t num_bytes, int shuffled, unsigned value, void* stream) {
-    // shuffled: 0 = address order; n > 0 = runs of n chunks (a power of two) in a scrambled order
-    return guarded([&] {
-        load_kernels(nullptr);
-        EP_HOST_ASSERT(dst != nullptr and ((uintptr_t)dst & 15) == 0);
-        EP_HOST_ASSERT(num_bytes > 0 and num_bytes % 4096 == 0 and num_bytes / 4096 <= INT32_MAX);
-        const unsigned chunks = (unsigned)(num_bytes / 4096);
-        EP_HOST_ASSERT(shuffled >= 0 and (shuffled & (shuffled - 1)) == 0);
-        EP_HOST_ASSERT(not shuffled or ((chunks & (chunks - 1)) == 0 and (unsigned)shuffled <= chunks));   // powers of two
-        EpCalibArgs ca = {dst, chunks, value, (unsigned)std::max(1, shuffled), 0u};
-        launch(shuffled ? g_k.calib_fill_shuffled : g_k.calib_fill, chunks, 256, 0, stream, ca);
-    });
-}
 
 int ep_fp8_selftest(uint64_t first, uint64_t count, float limit, uint64_t out[2]) {
     return guarded([&] {
@@ -1055,7 +1035,6 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* b, const ep_dispatch_epilogue_args_
         const unsigned grid = (unsigned)sa.num_row_blocks + pad_blocks;
         if (grid > 0) {
             hipFunction_t fn = quantise_here ? (g_fp8_hw ? g_k.scatter_quant : g_k.scatter_quant_sw) : g_k.scatter_copy;
-            if (quantise_here and g_stores_only) fn = g_k.scatter_quant_stores_only;
             launch(fn, grid, EP_ROW_THREADS, 0, a.stream, sa);
         }
         if (sf_columns and num_expanded > 0) {

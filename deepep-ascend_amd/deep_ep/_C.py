@@ -89,9 +89,6 @@ _ep_host_cvt = _sig('ep_host_f32_to_e4m3fn', None, ctypes.c_void_p, ctypes.c_voi
 _ep_selftest = _sig('ep_fp8_selftest', ctypes.c_int, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float,
                     ctypes.POINTER(ctypes.c_uint64))
 _ep_set_hw = _sig('ep_set_fp8_hw_convert', None, ctypes.c_int)
-_ep_calib_fill = _sig('ep_calibrate_fill', ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint,
-                      ctypes.c_void_p)
-_ep_set_stores_only = _sig('ep_set_calibration_stores_only', None, ctypes.c_int)
 _ep_create = _sig('ep_buffer_create', ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64,
                   ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p))
 _ep_destroy = _sig('ep_buffer_destroy', ctypes.c_int, ctypes.c_void_p)
@@ -241,18 +238,6 @@ def fp8_selftest(first: int, count: int, limit: float) -> Tuple[int, int]:
 
 def set_fp8_hw_convert(enable: bool) -> None:
     _ep_set_hw(int(enable))
-
-
-def calibrate_fill(dst: torch.Tensor, shuffled: int = 0, value: int = 0) -> None:
-    """Calibration write over the whole of `dst` (a multiple of 4 KiB) on the current stream: one 4 KiB chunk per
-    workgroup, in address order, or with runs of `shuffled` chunks in a scrambled order (powers of two)."""
-    init_jit()
-    _check(_ep_calib_fill(dst.data_ptr(), dst.numel() * dst.element_size(), int(shuffled), value, _stream()))
-
-
-def set_calibration_stores_only(enable: bool) -> None:
-    """Calibration: the fused-quantising copy kernel runs without its loads of x (outputs are garbage)."""
-    _ep_set_stores_only(int(enable))
 
 
 def set_combine_blocks_per_cu(num_blocks: int) -> None:

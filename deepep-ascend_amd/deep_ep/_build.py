@@ -3,6 +3,8 @@
   deep_ep/lib/ep_kernels.hsaco     device code object   (hipcc --genco)
   deep_ep/lib/libdeep_ep_hip.so    host runtime, C ABI  (hipcc -shared)
   deep_ep/lib/abi_client           a plain-C caller of the C ABI, used by the tests  (gcc)
+  ep_calib/lib/ep_calib.hsaco      calibration kernels of the benchmarks (not part of the product)
+  ep_calib/lib/libdeep_ep_calib.so their host side, C ABI of include/deep_ep_calib.h
 
 hipcc cross-compiles, so this runs on a machine without a GPU.  `python deepep-ascend_amd/deep_ep/_build.py`.
 """
@@ -13,6 +15,7 @@ import sys
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(PKG), 'csrc')
 LIB = os.path.join(PKG, 'lib')
+CALIB_LIB = os.path.join(os.path.dirname(PKG), 'ep_calib', 'lib')
 HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
 
 DEVICE_FLAGS = [
@@ -37,6 +40,10 @@ def build(verbose: bool = True) -> None:
     os.makedirs(LIB, exist_ok=True)
     run([HIPCC, *DEVICE_FLAGS, '-o', os.path.join(LIB, 'ep_kernels.hsaco'), os.path.join(CSRC, 'ep_kernels.hip')])
     run([HIPCC, *HOST_FLAGS, '-o', os.path.join(LIB, 'libdeep_ep_hip.so'), os.path.join(CSRC, 'ep_runtime.cpp')])
+    os.makedirs(CALIB_LIB, exist_ok=True)
+    run([HIPCC, *DEVICE_FLAGS, '-o', os.path.join(CALIB_LIB, 'ep_calib.hsaco'), os.path.join(CSRC, 'ep_calib.hip')])
+    run([HIPCC, '-shared', '-fPIC', '-O2', '-std=c++17', '-Wall', '-o', os.path.join(CALIB_LIB, 'libdeep_ep_calib.so'),
+         os.path.join(CSRC, 'ep_calib.cpp')])
     run(['gcc', *C_CLIENT_FLAGS, '-o', os.path.join(LIB, 'abi_client'), os.path.join(CSRC, 'abi_client.c'),
          f'-L{LIB}', '-ldeep_ep_hip', f'-L{ROCM}/lib', '-lamdhip64', '-Wl,-rpath,$ORIGIN', f'-Wl,-rpath,{ROCM}/lib'])
 

@@ -79,16 +79,6 @@ int ep_fp8_selftest(uint64_t first, uint64_t count, float limit, uint64_t out[2]
 /* 1: hardware v_cvt_pk_fp8_f32 (default), 0: integer conversion. */
 void ep_set_fp8_hw_convert(int enable);
 
-/* Calibration of the store path, for benchmarks (no counterpart in the reference).
- * ep_calibrate_fill: num_bytes / 4096 workgroups each write one 4 KiB chunk of dst with one 16-byte
- * non-temporal store per thread, in address order (shuffled = 0) or with runs of `shuffled` consecutive
- * chunks in a scrambled order (shuffled and the chunk count powers of two).  ep_set_calibration_stores_only(1): from then on the fused-quantising copy
- * kernel of ep_dispatch_epilogue_launch runs without its loads of x (same tasks, same stores to the same
- * slots, arbitrary payload): the price of the kernel's store pattern alone.  Outputs are garbage while it
- * is on. */
-int ep_calibrate_fill(void* dst, int64_t num_bytes, int shuffled, unsigned value, void* stream);
-void ep_set_calibration_stores_only(int enable);
-
 /* ---- buffer ---------------------------------------------------------------------------------- */
 
 /* One hipMalloc'd, zero-filled arena = workspace || buffer (num_bytes) || lb storage

@@ -206,3 +206,25 @@ def test_bench_refuses_more_than_one_gpu():
                        timeout=120)
     assert r.returncode == 2
     assert 'one GPU' in r.stderr and r.stdout.strip() == ''
+
+
+def test_calibration_rig_is_a_library_of_its_own(de):
+    """The benchmarks' calibration kernels live in their own library and code object: the product exports and
+    ships none of them, and the calibration library exports what its header declares."""
+    calib_dir = os.path.join(ROOT, 'deepep-ascend_amd', 'ep_calib', 'lib')
+    text = re.sub(r'/\*.*?\*/', '', open(os.path.join(ROOT, 'include', 'deep_ep_calib.h')).read(), flags=re.S)
+    names = sorted(set(re.findall(r'\b(ep_calib_[a-z0-9_]+)\s*\(', text)))
+    assert len(names) >= 6
+    calib = ctypes.CDLL(os.path.join(calib_dir, 'libdeep_ep_calib.so'))
+    product = ctypes.CDLL(LIB)
+    for n in names:
+        assert hasattr(calib, n), n
+        assert not hasattr(product, n), n
+    for gone in ('ep_calibrate_fill', 'ep_set_calibration_stores_only'):
+        assert not hasattr(product, gone), gone
+    blob = open(os.path.join(os.path.dirname(LIB), 'ep_kernels.hsaco'), 'rb').read()
+    assert b'ep_calib' not in blob and b'stores_only' not in blob
+    cblob = open(os.path.join(calib_dir, 'ep_calib.hsaco'), 'rb').read()
+    for k in (b'ep_calib_fill', b'ep_calib_fronts', b'ep_calib_mixed', b'ep_calib_scatter_stores_only', b'ep_calib_read_rows',
+              b'ep_calib_ordered_steered', b'ep_calib_copy_ordered_flat', b'gfx950'):
+        assert k in cblob, k
