@@ -3,10 +3,11 @@
 It exposes the names the reference's pybind module `deep_ep._C` exports for the EP path
 (csrc/python_api.cpp:18-74): `EventHandle`, `EPBuffer` with `.dispatch(27 args)` /
 `.combine(14 args)`, `calculate_ep_buffer_size`, the alignment getters, `topk_idx_t` and the
-runtime-configuration functions.  Torch tensors are only plumbing here: this module allocates
-outputs and passes raw device pointers plus the current HIP stream to the library.  There is no
-CPU or torch fallback: if the library or its code object is missing, importing or using this
-module raises.
+runtime-configuration functions.  Torch tensors are only plumbing here.  The two hot calls,
+`EPBuffer.dispatch` and `EPBuffer.combine`, are compiled (`_native`, csrc/python_api.cpp: pybind11 over
+the C ABI, as the reference's own binding is); everything else goes through ctypes.  There is no CPU
+or torch fallback: if the library, its code object or the compiled binding is missing, importing or
+using this module raises.
 """
 import ctypes
 import os
@@ -21,6 +22,12 @@ if not os.path.exists(_LIB_PATH):
     raise ImportError(f'{_LIB_PATH} is missing: build the native library first (python deepep-ascend_amd/deep_ep/_build.py)')
 
 _lib = ctypes.CDLL(_LIB_PATH)
+
+try:
+    from . import _native
+except ImportError as e:       # pragma: no cover
+    raise ImportError(f'the compiled binding deep_ep._native is missing or does not load ({e}): build it first '
+                      '(python deepep-ascend_amd/deep_ep/_build.py)') from e
 
 
 class _Tensor(ctypes.Structure):
@@ -111,8 +118,8 @@ _ep_dispatch_static = _sig('ep_dispatch_static_launch', ctypes.c_int, ctypes.POI
 _ep_combine = _sig('ep_combine_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_CombineArgs), ctypes.c_int)
 
 
-class EPException(RuntimeError):
-    """Raised for contract violations and runtime failures reported by the native library."""
+# Raised for contract violations and runtime failures reported by the native library (a RuntimeError).
+EPException = _native.EPException
 
 
 def _check(rc: int) -> None:
@@ -308,6 +315,12 @@ class EPBuffer(BufferBase):
         _check(_ep_create(rank_idx, num_ranks, num_bytes, num_lb_bytes, num_cpu_timeout_secs, num_gpu_timeout_secs,
                           ctypes.byref(handle)))
         self._h = handle
+        self._native = _native.Buffer(handle.value, rank_idx, num_ranks)
+        # the hot calls are the compiled binding's: dispatch(27 args, fused_fp8_quant=) in the argument order of
+        # csrc/buffers/ep.hpp:89-112, combine(14 args, apply_weights=) in that of csrc/buffers/ep.hpp:412-425; both
+        # return (result or None, EventHandle or None, deferred epilogue or None)
+        self.dispatch = self._native.dispatch
+        self.combine = self._native.combine
         self.connected = False
         self.device = torch.device('cuda', torch.cuda.current_device())
         self.context = Context(rank_idx, num_ranks)
@@ -324,6 +337,7 @@ class EPBuffer(BufferBase):
         if self.destroyed:
             raise EPException('Assertion exception (_C.py): not destroyed')
         self.lb_storage = None
+        self._native.invalidate()
         _check(_ep_destroy(self._h))
         self._h = None
         self.destroyed = True
@@ -349,10 +363,12 @@ class EPBuffer(BufferBase):
         if arena_bases is None:
             _check(_ep_set_peers(self._h, None, 0))
             self.connected = False
+            self._native.set_connected(False)
             return
         table = (ctypes.c_void_p * len(arena_bases))(*arena_bases)
         _check(_ep_set_peers(self._h, table, len(arena_bases)))
         self.connected = True
+        self._native.set_connected(True)
 
     @staticmethod
     def connect(runtimes) -> None:
@@ -362,6 +378,7 @@ class EPBuffer(BufferBase):
         _check(_ep_connect(handles, len(runtimes)))
         for r in runtimes:
             r.connected = True
+            r._native.set_connected(True)
 
     def region(self, which: int) -> Tuple[int, int]:
         n = ctypes.c_int64()
@@ -381,237 +398,6 @@ class EPBuffer(BufferBase):
 
     def lb_reduce_grads(self, *args, **kwargs):
         raise EPException('Assertion exception: EPBuffer::lb_reduce_grads is not implemented')
-
-    # ---- dispatch (argument order of csrc/buffers/ep.hpp:89-112) ----
-    def dispatch(self, x, sf, topk_idx, topk_weights, cumulative_local_expert_recv_stats,
-                 cached_num_recv_tokens, cached_num_expanded_tokens, cached_num_recv_tokens_per_expert_list,
-                 cached_psum_num_recv_tokens_per_rank, cached_psum_num_recv_tokens_per_expert,
-                 cached_num_unaligned_recv_tokens_per_expert, cached_dst_buffer_slot_idx, cached_dst_gsge_idx,
-                 cached_recv_src_metadata, num_max_tokens_per_rank, num_experts, expert_alignment, num_ai_cores,
-                 previous_event, async_with_compute_stream, allocate_on_comm_stream, do_handle_copy, do_cpu_sync,
-                 do_expand, do_zero_padding, use_col_major_sf, defer_epilogue, fused_fp8_quant=False):
-        if self.destroyed:
-            raise EPException('Assertion exception (_C.py): not destroyed')
-        if previous_event is not None:
-            previous_event.current_stream_wait()       # the launches below are ordered behind it
-        if not do_expand:
-            raise EPException('Assertion exception (_C.py): do_expand')
-        if do_handle_copy:
-            raise EPException('Assertion exception (_C.py): not do_handle_copy')
-        if num_ai_cores <= 0:
-            raise EPException('Assertion exception (_C.py): num_ai_cores > 0')
-        cached_mode = cached_num_recv_tokens is not None
-        if cached_mode:
-            for item in (cached_num_expanded_tokens, cached_num_recv_tokens_per_expert_list,
-                         cached_psum_num_recv_tokens_per_rank, cached_psum_num_recv_tokens_per_expert,
-                         cached_num_unaligned_recv_tokens_per_expert, cached_dst_buffer_slot_idx,
-                         cached_dst_gsge_idx, cached_recv_src_metadata):
-                if item is None:
-                    raise EPException('Assertion exception (_C.py): cached handle field has a value')
-        if x.dim() != 2 or topk_idx.dim() != 2:
-            raise EPException('Assertion exception (_C.py): x.dim() == 2 and topk_idx.dim() == 2')
-        num_tokens, hidden = x.shape
-        num_topk = topk_idx.size(1)
-        num_local_experts = num_experts // self.num_ranks
-        dev = x.device
-
-        def ints(*shape):
-            return torch.empty(shape, dtype=torch.int32, device=dev)
-
-        if cached_mode:
-            psum_rank, psum_expert = cached_psum_num_recv_tokens_per_rank, cached_psum_num_recv_tokens_per_expert
-            unaligned = cached_num_unaligned_recv_tokens_per_expert
-            dst_slot, dst_gsge = cached_dst_buffer_slot_idx, cached_dst_gsge_idx
-        else:
-            psum_rank, psum_expert, unaligned = ints(self.num_ranks), ints(num_local_experts), ints(num_local_experts)
-            dst_slot, dst_gsge = ints(num_tokens, num_topk), ints(num_tokens, num_topk)
-
-        a = _DispatchArgs()
-        a.x, a.sf = _desc(x), _desc(sf, two_byte_packs=True)
-        a.topk_idx, a.topk_weights = _desc(topk_idx), _desc(topk_weights)
-        a.cumulative_local_expert_recv_stats = _desc(cumulative_local_expert_recv_stats)
-        a.psum_num_recv_tokens_per_rank, a.psum_num_recv_tokens_per_expert = _desc(psum_rank), _desc(psum_expert)
-        a.num_unaligned_recv_tokens_per_expert = _desc(unaligned)
-        a.dst_buffer_slot_idx, a.dst_gsge_idx = _desc(dst_slot), _desc(dst_gsge)
-        a.num_max_tokens_per_rank, a.num_experts, a.expert_alignment = num_max_tokens_per_rank, num_experts, expert_alignment
-        a.cached_mode, a.do_cpu_sync, a.fused_fp8_quant = int(cached_mode), int(do_cpu_sync), int(fused_fp8_quant)
-        a.stream = _stream()
-        _check(_ep_dispatch(self._h, ctypes.byref(a)))
-        # the epilogue below belongs to this launch: the library refuses it once a later dispatch has
-        # taken over the buffer's workspace
-        stamp = _ep_stamp(self._h)
-
-        keep_alive = (x, sf, topk_idx, topk_weights, psum_rank, psum_expert)
-
-        def epilogue():
-            # the descriptors hold raw pointers: the inputs stay referenced until the copy kernel is enqueued
-            assert keep_alive is not None
-            per_expert_list: List[int] = []
-            partitioned = self.num_ranks > 1
-            # rows that can arrive: this partition's own tokens, or everybody's when the partitions form a node
-            rows_bound = self.num_ranks * num_max_tokens_per_rank if self.connected else num_tokens
-            recv_src_metadata = None
-            if partitioned and not cached_mode:
-                # receive side: count and rank the rows that arrived in this partition's regions
-                c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
-                _check(_ep_worst(self._h, num_max_tokens_per_rank, num_topk, num_experts, expert_alignment,
-                                 ctypes.byref(c_recv), ctypes.byref(c_exp)))
-                recv_src_metadata = ints(rows_bound if do_cpu_sync else c_recv.value, num_topk + 2)
-                r = _DispatchRecvArgs()
-                r.psum_num_recv_tokens_per_rank, r.psum_num_recv_tokens_per_expert = a.psum_num_recv_tokens_per_rank, \
-                    a.psum_num_recv_tokens_per_expert
-                r.num_unaligned_recv_tokens_per_expert = a.num_unaligned_recv_tokens_per_expert
-                r.cumulative_local_expert_recv_stats = a.cumulative_local_expert_recv_stats
-                r.recv_src_metadata = _desc(recv_src_metadata)
-                r.hidden_bytes = hidden * (1 if fused_fp8_quant else x.element_size())
-                r.num_sf_packs = 2 * ((hidden + 127) // 128) if fused_fp8_quant else (sf.size(1) if sf is not None else 0)
-                r.num_topk, r.num_max_tokens_per_rank = num_topk, num_max_tokens_per_rank
-                r.num_experts, r.expert_alignment = num_experts, expert_alignment
-                r.do_cpu_sync = int(do_cpu_sync)
-                r.dispatch_stamp = stamp
-                r.stream = _stream()
-                _check(_ep_dispatch_recv(self._h, ctypes.byref(r)))
-
-            def wait_counts():
-                c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
-                c_list = (ctypes.c_int * max(1, num_local_experts))()
-                _check(_ep_wait(self._h, ctypes.byref(c_recv), ctypes.byref(c_exp), c_list))
-                return c_recv.value, c_exp.value, c_list[:num_local_experts]       # (a slice of a ctypes array is a list)
-
-            if cached_mode:
-                num_recv, num_expanded = cached_num_recv_tokens, cached_num_expanded_tokens
-                per_expert_list = cached_num_recv_tokens_per_expert_list
-                alloc_recv, alloc_expanded = num_recv, num_expanded
-            elif do_cpu_sync and self.connected:
-                # a node: the bound over every partition's tokens is far above what arrives; wait for the counts
-                num_recv, num_expanded, per_expert_list = wait_counts()
-                alloc_recv, alloc_expanded = num_recv, num_expanded
-                recv_src_metadata = recv_src_metadata[:num_recv]
-            elif do_cpu_sync:
-                # Exact sizes come from the host count page, but waiting for it here would leave the GPU
-                # idle between the layout kernels and the copy.  Allocate for this call's upper bound,
-                # enqueue the copy, and read the counts while it runs; the results are narrowed below.
-                alloc_recv = num_tokens
-                alloc_expanded = num_tokens * min(num_topk, num_local_experts) + (expert_alignment - 1) * num_local_experts
-                alloc_expanded = -(-alloc_expanded // expert_alignment) * expert_alignment
-                num_recv = num_expanded = None
-            else:
-                c_recv, c_exp = ctypes.c_int(), ctypes.c_int()
-                _check(_ep_worst(self._h, num_max_tokens_per_rank, num_topk, num_experts, expert_alignment,
-                                 ctypes.byref(c_recv), ctypes.byref(c_exp)))
-                num_recv, num_expanded = c_recv.value, c_exp.value
-                alloc_recv, alloc_expanded = num_recv, num_expanded
-
-            out_dtype = torch.float8_e4m3fn if fused_fp8_quant else x.dtype
-            recv_x = torch.empty((alloc_expanded, hidden), dtype=out_dtype, device=dev)
-            recv_sf = None
-            if fused_fp8_quant or sf is not None:
-                sf_cols = (hidden + 127) // 128 if fused_fp8_quant else sf.size(1)
-                sf_dtype = torch.float32 if fused_fp8_quant else sf.dtype
-                sf_staging = None
-                if use_col_major_sf:
-                    # scale rows go to a staging tensor, a tiled kernel of the library turns them into columns
-                    sf_staging = torch.empty((alloc_expanded, sf_cols), dtype=sf_dtype, device=dev)
-                    sf_storage = torch.empty((sf_cols * alloc_expanded,), dtype=sf_dtype, device=dev)
-                    recv_sf = sf_storage.as_strided((alloc_expanded, sf_cols), (1, alloc_expanded))
-                else:
-                    recv_sf = torch.empty((alloc_expanded, sf_cols), dtype=sf_dtype, device=dev)
-            recv_topk_weights = None
-            if topk_weights is not None:
-                recv_topk_weights = torch.empty((alloc_expanded,), dtype=topk_weights.dtype, device=dev)
-            if cached_mode:
-                recv_src_metadata = cached_recv_src_metadata
-                if recv_src_metadata.dim() != 2 or recv_src_metadata.size(0) != num_recv:
-                    raise EPException('Assertion exception (_C.py): recv_src_metadata.size(0) == num_recv_tokens')
-            elif recv_src_metadata is None:
-                recv_src_metadata = ints(alloc_recv, num_topk + 2)
-
-            e = _DispatchEpilogueArgs()
-            e.x, e.sf, e.topk_weights = a.x, a.sf, a.topk_weights
-            e.psum_num_recv_tokens_per_rank = a.psum_num_recv_tokens_per_rank
-            e.psum_num_recv_tokens_per_expert = a.psum_num_recv_tokens_per_expert
-            e.recv_x, e.recv_sf = _desc(recv_x), _desc(recv_sf, two_byte_packs=not fused_fp8_quant)
-            if recv_sf is not None:
-                e.recv_sf_staging = _desc(sf_staging, two_byte_packs=not fused_fp8_quant)
-            e.recv_topk_weights, e.recv_src_metadata = _desc(recv_topk_weights), _desc(recv_src_metadata)
-            e.num_topk, e.num_max_tokens_per_rank = num_topk, num_max_tokens_per_rank
-            e.num_experts, e.expert_alignment = num_experts, expert_alignment
-            e.cached_mode, e.do_zero_padding = int(cached_mode), int(do_zero_padding)
-            e.fused_fp8_quant = int(fused_fp8_quant)
-            # sizes still unknown on the host: the column stride is the row count the device computed
-            e.recv_sf_layout = (2 if num_recv is None else 1) if use_col_major_sf else 0
-            e.stream = _stream()
-            e.dispatch_stamp = stamp
-            _check(_ep_dispatch_epi(self._h, ctypes.byref(e)))
-
-            if num_recv is None:
-                num_recv, num_expanded, per_expert_list = wait_counts()
-                if num_recv > alloc_recv or num_expanded > alloc_expanded:
-                    raise EPException('Assertion exception (_C.py): received counts exceed this call\'s bound')
-                recv_x = recv_x[:num_expanded]
-                if recv_sf is not None and use_col_major_sf:
-                    recv_sf = sf_storage.as_strided((num_expanded, sf_cols), (1, num_expanded))
-                elif recv_sf is not None:
-                    recv_sf = recv_sf[:num_expanded]
-                recv_topk_weights = recv_topk_weights[:num_expanded] if recv_topk_weights is not None else None
-                recv_src_metadata = recv_src_metadata[:num_recv]
-
-            return (recv_x, recv_sf, recv_topk_weights, num_recv, num_expanded, per_expert_list,
-                    psum_rank, psum_expert, unaligned, recv_src_metadata, dst_slot, dst_gsge)
-
-        if defer_epilogue:
-            if not async_with_compute_stream:
-                raise EPException('Assertion exception (_C.py): async_with_compute_stream')
-            return None, EventHandle(), epilogue
-        result = epilogue()
-        return result, (EventHandle() if async_with_compute_stream else None), None
-
-    # ---- combine (argument order of csrc/buffers/ep.hpp:412-425) ----
-    def combine(self, x, topk_weights, bias_0, bias_1, src_metadata, combined_topk_idx,
-                psum_num_recv_tokens_per_rank, num_experts, num_max_tokens_per_rank, num_sms, previous_event,
-                async_with_compute_stream, allocate_on_comm_stream, defer_epilogue, apply_weights=False):
-        if self.destroyed:
-            raise EPException('Assertion exception (_C.py): not destroyed')
-        if previous_event is not None:
-            previous_event.current_stream_wait()
-        if num_sms <= 0:
-            raise EPException('Assertion exception (_C.py): num_sms > 0')
-        if x.dim() != 2 or combined_topk_idx.dim() != 2:
-            raise EPException('Assertion exception (_C.py): x.dim() == 2 and combined_topk_idx.dim() == 2')
-        dev = x.device
-        hidden = x.size(1)
-        num_combined_tokens, num_topk = combined_topk_idx.shape
-
-        c = _CombineArgs()
-        c.x, c.topk_weights, c.bias_0, c.bias_1 = _desc(x), _desc(topk_weights), _desc(bias_0), _desc(bias_1)
-        c.src_metadata, c.combined_topk_idx = _desc(src_metadata), _desc(combined_topk_idx)
-        c.psum_num_recv_tokens_per_rank = _desc(psum_num_recv_tokens_per_rank)
-        c.num_experts, c.num_max_tokens_per_rank = num_experts, num_max_tokens_per_rank
-        c.apply_weights = int(apply_weights)
-        c.stream = _stream()
-        _check(_ep_combine(self._h, ctypes.byref(c), 0))           # owner side (nothing to do for one partition)
-
-        keep_alive = (x, topk_weights, bias_0, bias_1, src_metadata, combined_topk_idx, psum_num_recv_tokens_per_rank)
-
-        def epilogue():
-            # the descriptors hold raw pointers: the tensors stay referenced until the reduce is enqueued
-            assert keep_alive is not None
-            combined_x = torch.empty((num_combined_tokens, hidden), dtype=x.dtype, device=dev)
-            combined_topk_weights = None
-            if topk_weights is not None:
-                combined_topk_weights = torch.empty((num_combined_tokens, num_topk), dtype=topk_weights.dtype,
-                                                    device=dev)
-            c.combined_x, c.combined_topk_weights = _desc(combined_x), _desc(combined_topk_weights)
-            c.stream = _stream()
-            _check(_ep_combine(self._h, ctypes.byref(c), 1))       # token side
-            return combined_x, combined_topk_weights
-
-        if defer_epilogue:
-            if not async_with_compute_stream:
-                raise EPException('Assertion exception (_C.py): async_with_compute_stream')
-            return None, EventHandle(), epilogue
-        result = epilogue()
-        return result, (EventHandle() if async_with_compute_stream else None), None
 
 
 def barrier(context, with_cpu_sync: bool = False, sequential: bool = True, wait_comm_stream: bool = True) -> None:

@@ -2,6 +2,7 @@
 
   deep_ep/lib/ep_kernels.hsaco     device code object   (hipcc --genco)
   deep_ep/lib/libdeep_ep_hip.so    host runtime, C ABI  (hipcc -shared)
+  deep_ep/_native.*.so             compiled Python binding of dispatch/combine over that C ABI  (g++, pybind11 + torch headers)
   deep_ep/lib/abi_client           a plain-C caller of the C ABI, used by the tests  (gcc)
   ep_calib/lib/ep_calib.hsaco      calibration kernels of the benchmarks (not part of the product)
   ep_calib/lib/libdeep_ep_calib.so their host side, C ABI of include/deep_ep_calib.h
@@ -31,6 +32,21 @@ ROCM = os.environ.get('ROCM_PATH', '/opt/rocm')
 C_CLIENT_FLAGS = ['-std=c11', '-O1', '-Wall', '-D__HIP_PLATFORM_AMD__', f'-I{ROCM}/include']
 
 
+def binding_command():
+    """g++ line of the compiled binding: torch's headers and libraries (ROCm build), its bundled pybind11."""
+    import sysconfig
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    inc, tlib = os.path.join(tdir, 'include'), os.path.join(tdir, 'lib')
+    out = os.path.join(PKG, '_native' + sysconfig.get_config_var('EXT_SUFFIX'))
+    return ['g++', '-O2', '-std=c++17', '-shared', '-fPIC', '-fvisibility=hidden', '-Wall', '-Wno-unused-function',
+            f'-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}', '-DUSE_ROCM', '-D__HIP_PLATFORM_AMD__=1',
+            f'-I{inc}', f'-I{inc}/torch/csrc/api/include', f'-I{ROCM}/include', f'-I{sysconfig.get_paths()["include"]}',
+            os.path.join(CSRC, 'python_api.cpp'), '-o', out,
+            f'-L{LIB}', '-ldeep_ep_hip', f'-L{tlib}', '-ltorch_python', '-ltorch', '-ltorch_cpu', '-ltorch_hip', '-lc10', '-lc10_hip',
+            '-Wl,-rpath,$ORIGIN/lib', f'-Wl,-rpath,{tlib}']
+
+
 def run(cmd):
     print(' '.join(cmd), flush=True)
     subprocess.check_call(cmd)
@@ -40,6 +56,7 @@ def build(verbose: bool = True) -> None:
     os.makedirs(LIB, exist_ok=True)
     run([HIPCC, *DEVICE_FLAGS, '-o', os.path.join(LIB, 'ep_kernels.hsaco'), os.path.join(CSRC, 'ep_kernels.hip')])
     run([HIPCC, *HOST_FLAGS, '-o', os.path.join(LIB, 'libdeep_ep_hip.so'), os.path.join(CSRC, 'ep_runtime.cpp')])
+    run(binding_command())
     os.makedirs(CALIB_LIB, exist_ok=True)
     run([HIPCC, *DEVICE_FLAGS, '-o', os.path.join(CALIB_LIB, 'ep_calib.hsaco'), os.path.join(CSRC, 'ep_calib.hip')])
     run([HIPCC, '-shared', '-fPIC', '-O2', '-std=c++17', '-Wall', '-o', os.path.join(CALIB_LIB, 'libdeep_ep_calib.so'),

@@ -41,21 +41,21 @@ class EPHandle:
             output (upper bounds when the dispatch did not sync with the host).
     """
 
-    _CALL_FIELDS = ('do_expand', 'num_experts', 'expert_alignment', 'num_max_tokens_per_rank', 'num_sms')
-    _LAYOUT_FIELDS = ('num_recv_tokens', 'num_expanded_tokens', 'num_recv_tokens_per_expert_list',
-                      'psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
-                      'num_unaligned_recv_tokens_per_expert', 'recv_src_metadata', 'dst_buffer_slot_idx',
-                      'dst_gsge_idx')
-
     def __init__(self, do_expand: bool, num_experts: int, expert_alignment: int, num_max_tokens_per_rank: int,
                  num_sms: int, topk_idx: torch.Tensor, num_recv_tokens: int, num_expanded_tokens: int,
                  num_recv_tokens_per_expert_list: list, psum_num_recv_tokens_per_rank: torch.Tensor,
                  psum_num_recv_tokens_per_expert: torch.Tensor, num_unaligned_recv_tokens_per_expert: torch.Tensor,
                  recv_src_metadata: torch.Tensor, dst_buffer_slot_idx: torch.Tensor, dst_gsge_idx: torch.Tensor):
         assert topk_idx is not None
-        given = locals()
-        for name in self._CALL_FIELDS + self._LAYOUT_FIELDS:
-            setattr(self, name, given[name])
+        self.do_expand, self.num_experts, self.expert_alignment = do_expand, num_experts, expert_alignment
+        self.num_max_tokens_per_rank, self.num_sms = num_max_tokens_per_rank, num_sms
+        self.num_recv_tokens, self.num_expanded_tokens = num_recv_tokens, num_expanded_tokens
+        self.num_recv_tokens_per_expert_list = num_recv_tokens_per_expert_list
+        self.psum_num_recv_tokens_per_rank = psum_num_recv_tokens_per_rank
+        self.psum_num_recv_tokens_per_expert = psum_num_recv_tokens_per_expert
+        self.num_unaligned_recv_tokens_per_expert = num_unaligned_recv_tokens_per_expert
+        self.recv_src_metadata = recv_src_metadata
+        self.dst_buffer_slot_idx, self.dst_gsge_idx = dst_buffer_slot_idx, dst_gsge_idx
         self.cached_recv_src_metadata_before_sort = None
         self._topk_idx = topk_idx
         # inference tensors carry no version counter
@@ -136,6 +136,7 @@ class EPBuffer(BufferBase):
         if os.environ.get('EP_BUFFER_DEBUG'):
             print(f'EP buffer of partition {rank_idx}/{num_ranks}: {num_bytes} bytes + {num_lb_bytes} bytes of storage')
 
+        self._num_compute_units = None
         self.runtime = _C.EPBuffer(rank_idx, num_ranks, self.hccl_comm_handle.get(), num_bytes, num_lb_bytes,
                                    use_huge1g_page, num_cpu_timeout_secs, num_gpu_timeout_secs, explicitly_destroy)
         self.context = self.runtime.context
@@ -171,7 +172,10 @@ class EPBuffer(BufferBase):
     def get_theoretical_num_sms(self, num_experts: int, num_topk: int, num_scaleout_topk: int = 0,
                                 rdma_gbs: float = 0, nvlink_gbs: float = 0,
                                 sm_read_gbs: float = 0, sm_write_gbs: float = 0) -> int:
-        return _C.get_num_ai_cores()
+        # launches size themselves; the figure only travels in the handle (asked of the device once)
+        if self._num_compute_units is None:
+            self._num_compute_units = _C.get_num_ai_cores()
+        return self._num_compute_units
 
     def get_theoretical_num_qps(self, num_sms: int) -> int:
         return 0

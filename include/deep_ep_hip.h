@@ -190,6 +190,13 @@ int ep_dispatch_wait_counts(ep_buffer_t* buf, int* num_recv_tokens, int* num_exp
 int ep_dispatch_worst_case_sizes(ep_buffer_t* buf, int num_max_tokens_per_rank, int num_topk, int num_experts,
                                  int expert_alignment, int* num_recv_tokens, int* num_expanded_tokens);
 
+/* recv_sf_layout of ep_dispatch_epilogue_args_t */
+enum ep_sf_layout {
+    EP_SF_LAYOUT_ROW_MAJOR = 0,
+    EP_SF_LAYOUT_COL_MAJOR = 1,
+    EP_SF_LAYOUT_COL_MAJOR_COUNTED = 2
+};
+
 typedef struct ep_dispatch_epilogue_args {
     ep_tensor_t x, sf, topk_weights;                    /* as given to ep_dispatch_launch */
     ep_tensor_t psum_num_recv_tokens_per_rank, psum_num_recv_tokens_per_expert;
