@@ -513,14 +513,14 @@ def main():
 
     # The timed region: K steps back to back.  Events on the launch stream split every step into its
     # dispatch phase (layout kernels, host count read, copy kernel) and its combine kernel.
-    marks = [tuple(torch.cuda.Event(enable_timing=True) for _ in range(3)) for _ in range(args.steps)]
+    # (two events a step: a step ends where the next one starts; one more event closes the last step)
+    marks = [tuple(torch.cuda.Event(enable_timing=True) for _ in range(2)) for _ in range(args.steps + 1)]
 
     def marked_step(m):
         m[0].record()
         r, _, rw, h, _ = dispatch()
         m[1].record()
         buf.combine(y, h, topk_weights=rw)
-        m[2].record()
 
     graph = None
     if args.graph:
@@ -535,14 +535,16 @@ def main():
         graph.replay() if graph is not None else step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for m in marks:
+    for m in marks[:-1]:
         graph.replay() if graph is not None else marked_step(m)
+    if graph is None:
+        marks[-1][0].record()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     loop_dispatch = loop_combine = None
     if graph is None:
-        loop_dispatch = sorted(m[0].elapsed_time(m[1]) * 1e3 for m in marks)
-        loop_combine = sorted(m[1].elapsed_time(m[2]) * 1e3 for m in marks)
+        loop_dispatch = sorted(m[0].elapsed_time(m[1]) * 1e3 for m in marks[:-1])
+        loop_combine = sorted(m[1].elapsed_time(n[0]) * 1e3 for m, n in zip(marks[:-1], marks[1:]))
 
     # Isolated samples: each kernel alone (the copy kernel as the epilogue of a deferred dispatch, and again as
     # what a cached dispatch enqueues).  Ten untimed launches, then --samples timed ones; before each a 1 GiB scratch buffer is rewritten, so no sample finds its inputs in
@@ -617,6 +619,26 @@ def main():
     avg = lambda v: sum(v) / len(v)  # noqa: E731
     med = lambda v: v[len(v) // 2]  # noqa: E731
     us_scatter = med(t_scatter)
+
+    def host_issue_us(n):
+        # What the calls cost on the host: a dispatch without the host's wait for the counts and a combine are only
+        # enqueued (outputs at their worst-case sizes), nothing waits for the GPU inside the bracket.
+        r0, _, rw0, h0, _ = buf.dispatch(xg, topk_idx=tg, topk_weights=wg, do_cpu_sync=False, **kw)
+        y_ws = torch.empty(((r0[0] if fp8 else r0).size(0), H), dtype=torch.bfloat16, device=dev)
+        del r0, rw0, h0
+        best = None
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
+            for _ in range(n):
+                r1, _, rw1, h1, _ = buf.dispatch(xg, topk_idx=tg, topk_weights=wg, do_cpu_sync=False, **kw)
+                buf.combine(y_ws, h1, topk_weights=rw1)
+            t_host = (time.perf_counter() - t_start) * 1e6 / n
+            best = t_host if best is None else min(best, t_host)
+        torch.cuda.synchronize()
+        return best
+
+    us_host = host_issue_us(20 if T * H >= (1 << 24) else 200)
     traffic, traffic_source = measured_traffic(args.workload) if not args.no_cpu_sync else ({}, 'not the profiled configuration')
 
     def roof(name, nbytes, samples):
@@ -679,6 +701,8 @@ def main():
             'dispatch_gbs': round(b_d / us_dispatch / 1e3, 1), 'dispatch_frac_hbm': round(b_d / us_dispatch / 1e3 / HBM_PEAK_GBS, 4),
             'combine_us': round(us_combine, 2), 'combine_gbs': round(b_c / us_combine / 1e3, 1),
             'combine_frac_hbm': round(b_c / us_combine / 1e3 / HBM_PEAK_GBS, 4),
+            # host time of the two calls (enqueue only: dispatch without host sync + combine; best of three loops)
+            'host_us': round(us_host, 2),
             'dispatch_bytes': b_d, 'combine_bytes': b_c, 'zero_padding_bytes_not_counted': pad_bytes,
             'scatter_gbs_incl_padding': round((b_d + pad_bytes) / us_scatter / 1e3, 1),
         },

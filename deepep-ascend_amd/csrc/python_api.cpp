@@ -5,6 +5,7 @@
 // contract and every launch lives behind the C ABI in libdeep_ep_hip.so.
 #include <torch/extension.h>
 
+#include <ATen/hip/EmptyTensor.h>
 #include <c10/hip/HIPStream.h>
 
 #include <memory>
@@ -86,9 +87,12 @@ py::object new_event() {
     return cls();
 }
 
-at::Tensor empty_i32(std::initializer_list<int64_t> shape, const at::Device& dev) {
-    return at::empty(shape, at::TensorOptions().dtype(at::kInt).device(dev));
+// Uninitialised device tensors straight from torch's caching allocator (what at::empty reaches through its
+// dispatcher).
+at::Tensor alloc(at::IntArrayRef shape, at::ScalarType dtype, const at::Device& dev) {
+    return at::Tensor(at::detail::empty_cuda(shape, dtype, dev, std::nullopt));
 }
+at::Tensor empty_i32(std::initializer_list<int64_t> shape, const at::Device& dev) { return alloc(shape, at::kInt, dev); }
 
 // What a dispatch call keeps until its copy epilogue has been enqueued (the descriptors hold raw pointers:
 // the tensors stay referenced here).
@@ -181,24 +185,23 @@ py::tuple run_dispatch_epilogue(DispatchState& s) {
         alloc_expanded = c_exp;
     }
 
-    const auto x_opts = s.x.options();
-    at::Tensor recv_x = at::empty({alloc_expanded, H}, s.fused ? x_opts.dtype(at::kFloat8_e4m3fn) : x_opts);
+    at::Tensor recv_x = alloc({alloc_expanded, H}, s.fused ? at::kFloat8_e4m3fn : s.x.scalar_type(), dev);
     OptTensor recv_sf, sf_staging, sf_storage, recv_w;
     int64_t sf_cols = 0;
     const bool has_sf = s.fused || s.sf.has_value();
     if (has_sf) {
         sf_cols = s.fused ? (H + 127) / 128 : s.sf->size(1);
-        const auto sf_opts = s.fused ? x_opts.dtype(at::kFloat) : s.sf->options();
+        const at::ScalarType sf_type = s.fused ? at::kFloat : s.sf->scalar_type();
         if (s.use_col_major_sf) {
             // scale rows go to a staging tensor, a tiled kernel of the library turns them into columns
-            sf_staging = at::empty({alloc_expanded, sf_cols}, sf_opts);
-            sf_storage = at::empty({sf_cols * alloc_expanded}, sf_opts);
+            sf_staging = alloc({alloc_expanded, sf_cols}, sf_type, dev);
+            sf_storage = alloc({sf_cols * alloc_expanded}, sf_type, dev);
             recv_sf = sf_storage->as_strided({alloc_expanded, sf_cols}, {1, alloc_expanded});
         } else {
-            recv_sf = at::empty({alloc_expanded, sf_cols}, sf_opts);
+            recv_sf = alloc({alloc_expanded, sf_cols}, sf_type, dev);
         }
     }
-    if (s.topk_weights.has_value()) recv_w = at::empty({alloc_expanded}, s.topk_weights->options());
+    if (s.topk_weights.has_value()) recv_w = alloc({alloc_expanded}, s.topk_weights->scalar_type(), dev);
     if (s.cached_mode) {
         meta = *s.cached_meta;
         if (meta.dim() != 2 || meta.size(0) != num_recv)
@@ -268,9 +271,10 @@ struct CombineState {
 };
 
 py::tuple run_combine_epilogue(CombineState& s) {
-    at::Tensor combined_x = at::empty({s.num_combined_tokens, s.hidden}, s.x.options());
+    at::Tensor combined_x = alloc({s.num_combined_tokens, s.hidden}, s.x.scalar_type(), s.x.device());
     OptTensor combined_w;
-    if (s.topk_weights.has_value()) combined_w = at::empty({s.num_combined_tokens, s.num_topk}, s.topk_weights->options());
+    if (s.topk_weights.has_value())
+        combined_w = alloc({s.num_combined_tokens, s.num_topk}, s.topk_weights->scalar_type(), s.x.device());
     s.c.combined_x = desc(combined_x);
     s.c.combined_topk_weights = desc(combined_w);
     s.c.stream = current_stream();
@@ -311,6 +315,7 @@ public:
         }
         if (x.dim() != 2 || topk_idx.dim() != 2)
             throw EpPyError("Assertion exception (python_api.cpp): x.dim() == 2 and topk_idx.dim() == 2");
+        if (!x.is_cuda()) throw EpPyError("every tensor handed to the EP kernels must live on the GPU");
         auto st = std::make_shared<DispatchState>();
         DispatchState& s = *st;
         s.buf = buf_;
@@ -345,9 +350,12 @@ public:
             s.cached_num_recv = *cached_num_recv_tokens;
             s.cached_num_expanded = *cached_num_expanded_tokens;
         } else {
-            s.psum_rank = empty_i32({num_ranks_}, dev);
-            s.psum_expert = empty_i32({s.num_local_experts}, dev);
-            s.unaligned = empty_i32({s.num_local_experts}, dev);
+            // the three count vectors share one allocation (each starts on a multiple of 64 bytes)
+            const int64_t r16 = (num_ranks_ + 15) / 16 * 16, e16 = (s.num_local_experts + 15) / 16 * 16;
+            at::Tensor counts = empty_i32({r16 + 2 * e16}, dev);
+            s.psum_rank = counts.narrow(0, 0, num_ranks_);
+            s.psum_expert = counts.narrow(0, r16, s.num_local_experts);
+            s.unaligned = counts.narrow(0, r16 + e16, s.num_local_experts);
             s.dst_slot = empty_i32({s.num_tokens, s.num_topk}, dev);
             s.dst_gsge = empty_i32({s.num_tokens, s.num_topk}, dev);
         }
@@ -397,6 +405,7 @@ public:
         EP_PY_ASSERT(num_sms > 0);
         if (x.dim() != 2 || combined_topk_idx.dim() != 2)
             throw EpPyError("Assertion exception (python_api.cpp): x.dim() == 2 and combined_topk_idx.dim() == 2");
+        if (!x.is_cuda()) throw EpPyError("every tensor handed to the EP kernels must live on the GPU");
         auto st = std::make_shared<CombineState>();
         CombineState& s = *st;
         s.buf = buf_;
@@ -422,7 +431,9 @@ public:
         c.num_max_tokens_per_rank = num_max_tokens_per_rank;
         c.apply_weights = apply_weights ? 1 : 0;
         c.stream = current_stream();
-        check(ep_combine_launch(buf_, &c, 0));       // owner side (validates only, with one partition)
+        // owner side; with one partition it only validates, which the token side below repeats: then it is called
+        // only where the token side is deferred, so that a bad argument still fails at the call
+        if (num_ranks_ > 1 || defer_epilogue) check(ep_combine_launch(buf_, &c, 0));
 
         if (defer_epilogue) {
             if (!async_with_compute_stream) throw EpPyError("Assertion exception (python_api.cpp): async_with_compute_stream");

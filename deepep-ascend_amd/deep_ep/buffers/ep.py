@@ -228,7 +228,8 @@ class EPBuffer(BufferBase):
         Returns `(recv_x or (recv_x, recv_sf), None, recv_topk_weights, handle, event)`, or the
         `EventOverlap` alone when `defer_epilogue`.
         """
-        self._no_explicit_qps(num_qps)
+        if num_qps:
+            self._no_explicit_qps(num_qps)
         if do_handle_copy:
             raise AssertionError('`do_handle_copy` must be False; handle copying is no longer supported')
         if not do_expand:
@@ -248,11 +249,14 @@ class EPBuffer(BufferBase):
             topk_idx, num_sms, do_cpu_sync = handle.topk_idx, handle.num_sms, False
             cached_fields = tuple(getattr(handle, name) for name in self._RUNTIME_CACHED_ORDER)
         else:
-            num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, self.num_max_tokens_per_rank)
-            expert_alignment = value_or(expert_alignment, 1)
-            do_cpu_sync = value_or(do_cpu_sync, True)
-            num_sms = num_sms or self.get_theoretical_num_sms(num_experts, topk_idx.size(1))
-            cached_fields = (None,) * len(self._RUNTIME_CACHED_ORDER)
+            if num_max_tokens_per_rank is None:
+                num_max_tokens_per_rank = self.num_max_tokens_per_rank
+            if expert_alignment is None:
+                expert_alignment = 1
+            if do_cpu_sync is None:
+                do_cpu_sync = True
+            num_sms = num_sms or self._num_compute_units or self.get_theoretical_num_sms(num_experts, topk_idx.size(1))
+            cached_fields = self._NO_CACHED_FIELDS
 
         result, event, deferred = self.runtime.dispatch(
             payload, sf, topk_idx, topk_weights, cumulative_local_expert_recv_stats, *cached_fields,
@@ -280,6 +284,7 @@ class EPBuffer(BufferBase):
         overlap.register_hook_after_wait(lambda: finish(deferred(), False))
         return overlap
 
+    _NO_CACHED_FIELDS = (None,) * 9
     # order in which the native runtime takes the fields of a cached handle (csrc/buffers/ep.hpp:96-104)
     _RUNTIME_CACHED_ORDER = ('num_recv_tokens', 'num_expanded_tokens', 'num_recv_tokens_per_expert_list',
                              'psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
@@ -321,7 +326,8 @@ class EPBuffer(BufferBase):
 
         Returns `(combined_x, combined_topk_weights, event)`, or the `EventOverlap` alone.
         """
-        self._no_explicit_qps(num_qps)
+        if num_qps:
+            self._no_explicit_qps(num_qps)
         if handle.recv_src_metadata is None:
             raise AssertionError('the handle comes from a dispatch that ran its epilogue')
         bias_0, bias_1 = self._unpack_bias(bias)
