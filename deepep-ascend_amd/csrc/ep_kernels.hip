@@ -1195,12 +1195,14 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
     if (verbatim) {
         const int s1 = readlane(myslot, __builtin_ctzll(__ballot(myslot >= 0)));
         const u32x4* src = y + (int64_t)s1 * yvec;
-        for (int vb = lane; vb < nvec; vb += 16 * WAVE) {
+        // (the loop counter is the same in every lane: a row shorter than the wave still gets its weights)
+        for (int v0 = 0; v0 < nvec; v0 += 16 * WAVE) {
+            const int vb = v0 + lane;
             u32x4 d[16];
 #pragma unroll
             for (int u = 0; u < 16; ++u)
                 if (vb + u * WAVE < nvec) d[u] = __builtin_nontemporal_load(src + vb + u * WAVE);
-            if (vb == lane && lane < K && a.expanded_weights != nullptr) ((float*)(out_row + (a.hidden << 1)))[lane] = myw;
+            if (v0 == 0 && lane < K && a.expanded_weights != nullptr) ((float*)(out_row + (a.hidden << 1)))[lane] = myw;
 #pragma unroll
             for (int u = 0; u < 16; ++u)
                 if (vb + u * WAVE < nvec) stream_store<EP_COMBINE_ST_POL>(out + vb + u * WAVE, d[u]);

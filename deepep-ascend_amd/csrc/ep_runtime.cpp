@@ -7,6 +7,7 @@
 #include <dlfcn.h>
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
@@ -120,7 +121,7 @@ struct Kernels {
 
 std::mutex g_mutex;
 Kernels g_k;
-bool g_fp8_hw = true;
+std::atomic<bool> g_fp8_hw{true};
 // Workgroups of the single-partition combine kernel a CU holds at once, enforced through an unused dynamic LDS
 // allocation (0: no cap, the registers decide: 5 to 8; negative: chosen by top-k, below).  The gather is fastest
 // with about 150 KiB of row fetches in flight a CU (a wave fetches top-k x 2 KiB): more waves queue more fetches
@@ -130,7 +131,7 @@ bool g_fp8_hw = true;
 // and for the kernel that takes any top-k: top-1 best uncapped, top-3 at 6, top-5 at 5, top-7 to top-16 at 4.
 // A bias row is one more row a wave fetches: top-6 with one / two biases 326 311 329 336 / 358 350 373 377 at 2/3/4/5.
 // The two-phase kernels of the partitioned path do not react to it.
-int g_combine_blocks_per_cu = -1;
+std::atomic<int> g_combine_blocks_per_cu{-1};
 constexpr unsigned kLdsBytesPerCu = 160 * 1024;
 unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks, int hidden) {     // num_topk: rows a wave fetches, biases included
     int n = g_combine_blocks_per_cu;
@@ -143,11 +144,14 @@ unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks, int
         else if (specialised) n = num_topk <= 2 ? 0 : num_topk <= 4 ? 4 : 3;
         else n = num_topk <= 2 ? 0 : num_topk == 3 ? 6 : num_topk <= 5 ? 5 : 4;
     }
+    // a workgroup can ask for 64 KiB at most, which lets two of them into a CU: a cap of one cannot be enforced this
+    // way (it is served as two), and from 160 workgroups on a share of the LDS is too small to mean anything (no cap)
     if (n <= 0) return 0;
     const unsigned share = kLdsBytesPerCu / (unsigned)n;
+    if (share <= 1024u) return 0;
     return std::min(64u * 1024u, share - 1024u);       // n of them fit a CU, n + 1 do not
 }
-int g_fold_max_blocks = 256;    // up to this many layout workgroups the slot assignment sums the block counts itself
+std::atomic<int> g_fold_max_blocks{256};    // up to this many layout workgroups the slot assignment sums the block counts itself
 
 std::string library_dir() {
     Dl_info info;
@@ -1232,6 +1236,18 @@ ep_buffer* static_view_of_current_device() {
 }  // namespace
 
 void ep_static_scratch_init() { (void)static_view_of_current_device(); }
+
+// Bytes of the static scratch a single-partition dispatch of this shape carves: the header, then the column
+// totals, the count matrix, the slot map and the token -> row map, each rounded up to 64 ints (what
+// ep_dispatch_launch carves from a workspace, restated).
+extern "C" int64_t ep_dispatch_static_scratch_bytes(int num_tokens, int num_topk, int num_experts) {
+    if (num_tokens < 0 or num_topk <= 0 or num_experts <= 0) return -1;
+    auto a64 = [](int64_t n) { return align_up(std::max<int64_t>(n, 1), 64); };
+    const int64_t W = align_up((int64_t)num_experts + 1, 4);
+    const int64_t B = std::max<int64_t>(1, ceil_div(num_tokens, EP_TOKENS_PER_BLOCK));
+    return EP_WS_HEADER_BYTES + 4 * (a64(W) + a64(B * W) + a64((int64_t)num_tokens * num_topk) + a64(num_tokens));
+}
+extern "C" int64_t ep_dispatch_static_scratch_capacity(void) { return EP_STATIC_SCRATCH_BYTES; }
 
 extern "C" int ep_dispatch_static_launch(const ep_dispatch_args_t* d, const ep_dispatch_epilogue_args_t* e) {
     int rc = guarded([&] {

@@ -115,6 +115,8 @@ _ep_set_fold = _sig('ep_set_layout_fold_max_blocks', None, ctypes.c_int)
 _ep_set_combine_cap = _sig('ep_set_combine_blocks_per_cu', None, ctypes.c_int)
 _ep_dispatch_static = _sig('ep_dispatch_static_launch', ctypes.c_int, ctypes.POINTER(_DispatchArgs),
                            ctypes.POINTER(_DispatchEpilogueArgs))
+_ep_static_bytes = _sig('ep_dispatch_static_scratch_bytes', ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int)
+_ep_static_capacity = _sig('ep_dispatch_static_scratch_capacity', ctypes.c_int64)
 _ep_combine = _sig('ep_combine_launch', ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(_CombineArgs), ctypes.c_int)
 
 

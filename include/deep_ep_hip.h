@@ -168,7 +168,9 @@ void ep_set_layout_fold_max_blocks(int num_blocks);
 
 /* Tuning: workgroups (of 4 waves) of the single-partition combine kernel that a compute unit holds at once;
  * 0 lifts the cap, a negative value lets the library choose by top-k (the default: 3 at top-6 and top-8,
- * 4 at top-4, none at top-2 and for launches too small to fill the machine twice).  Results do not depend on it. */
+ * 4 at top-4, none at top-2 and for launches too small to fill the machine twice).  The cap is enforced through
+ * an LDS allocation: the smallest one that can be enforced is 2 (a request for 1 is served as 2), and values from
+ * 160 on mean no cap.  Results do not depend on it. */
 void ep_set_combine_blocks_per_cu(int num_blocks);
 
 /* More than one partition, non-cached dispatch: the receive side of launch_dispatch and the slot
@@ -228,14 +230,19 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* buf, const ep_dispatch_epilogue_arg
 
 /* A whole single-partition dispatch without a host sync (ep_dispatch_launch followed by
  * ep_dispatch_epilogue_launch, non-cached, do_cpu_sync = 0) that needs no ep_buffer and allocates
- * nothing: the layout scratch lives in a 4 MiB device array inside the library instead of a buffer's
- * arena.  It has no counterpart in the reference; it is for callers that cannot allocate (code under
- * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The caller passes every
- * input and output, the outputs sized by ep_dispatch_worst_case_sizes(NULL, ...);
- * epilogue_args->dispatch_stamp is ignored.  Fails with a clear message when the scratch the shape needs (about
- * 4 * (T*K + max_tokens + ceil(T/128) * (E + 64)) bytes) exceeds the array.  Results equal those of the
- * two calls it stands for.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
- * (different streams, or host threads) race; calls on one stream are ordered and safe. */
+ * nothing: the layout scratch lives in a device array inside the library (ep_dispatch_static_scratch_capacity()
+ * bytes, 4 MiB) instead of a buffer's arena.  It has no counterpart in the reference; it is for callers that
+ * cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * ep_init must have run on the device before the first such call: loading the code object and looking up the
+ * array's address do allocate, and ep_init is where they happen.  The caller passes every input and output, the
+ * outputs sized by ep_dispatch_worst_case_sizes(NULL, ...); epilogue_args->dispatch_stamp is ignored.  Fails
+ * with a clear message when the scratch the shape needs, ep_dispatch_static_scratch_bytes(T, K, E) =
+ * 4096 + 4 * (a64(W) + a64(B * W) + a64(T * K) + a64(T)) with W = E + 1 rounded up to 4, B = ceil(T / 128) (at
+ * least 1) and a64 rounding up to a multiple of 64, exceeds the array.  Results equal those of the two calls it
+ * stands for.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (different streams,
+ * or host threads) race; calls on one stream are ordered and safe. */
+int64_t ep_dispatch_static_scratch_bytes(int num_tokens, int num_topk, int num_experts);
+int64_t ep_dispatch_static_scratch_capacity(void);
 int ep_dispatch_static_launch(const ep_dispatch_args_t* args, const ep_dispatch_epilogue_args_t* epilogue_args);
 
 /* ---- combine --------------------------------------------------------------------------------- */

@@ -469,3 +469,46 @@ def test_node_rejects_scaled_rows_that_would_overlap():
     single.destroy()
     for b in bufs:
         b.destroy()
+
+
+def test_owner_side_whole_rows_shorter_than_a_wave_carry_all_their_weights():
+    """From 16384 metadata rows on the owner-side reduce takes whole rows per wave, and a row with a single local
+    slot is copied verbatim.  With rows of fewer 16-byte vectors than top-k positions (hidden 64, top-16) the
+    weight vector of such a row is wider than its payload: every position of it must still be written."""
+    R, max_tokens, H, E, K, A = 2, 8400, 64, 32, 16, 8
+    bufs = make_node(R, max_tokens, H, K, False)
+    Ts = [max_tokens, max_tokens - 100]
+    xs = [make_tokens(T, H, seed=50 + r) for r, T in enumerate(Ts)]
+    routing = [make_routing(T, E, K, seed=60 + r, masked=0.85) for r, T in enumerate(Ts)]     # mostly one local slot a row
+    topks, ws = [t for t, _ in routing], [w for _, w in routing]
+    rows = [bf16_bits(x).view(np.uint8).reshape(x.size(0), -1) for x in xs]
+    _, want = oracle_dispatch(rows, [None] * R, [t.numpy() for t in topks], [w.numpy() for w in ws], E, R, A, max_tokens)
+    outs = dispatch_all(bufs, [x.to(DEV) for x in xs], [t.to(DEV) for t in topks], [w.to(DEV) for w in ws],
+                        num_experts=E, num_max_tokens_per_rank=max_tokens, expert_alignment=A, do_expand=True,
+                        do_zero_padding=True, do_cpu_sync=False)
+    torch.cuda.synchronize()
+    handles = [o[3] for o in outs]
+    assert all(h.recv_src_metadata.size(0) >= 16384 for h in handles)          # the whole-row path is the one that runs
+    single = sum(int(((want[r]['lay']['recv_src_metadata'][:, :K] >= 0).sum(axis=1) == 1).sum()) for r in range(R))
+    assert single > 1000                                                       # and verbatim rows are many
+    g = torch.Generator().manual_seed(7)
+    ys = [torch.randn((outs[r][0].size(0), H), generator=g).to(torch.bfloat16) for r in range(R)]
+    # the combine buffers hold what earlier phases left: poison them, so that a position nobody writes shows
+    for b in bufs:
+        b.runtime.buffer_tensor().fill_(0x5A)
+    res = combine_all(bufs, [y.to(DEV) for y in ys], handles, [o[2] for o in outs], [None] * R)
+    torch.cuda.synchronize()
+    parts, wvecs = {}, {}
+    for r in range(R):
+        ne = want[r]['lay']['num_expanded_tokens']
+        p, wv = O.combine_partial(ys[r][:ne], torch.from_numpy(want[r]['w']), want[r]['lay']['recv_src_metadata'], R, r, max_tokens)
+        parts.update(p)
+        wvecs.update(wv)
+    for s in range(R):
+        ox, ow = O.combine_final(topks[s].numpy(), E, R, s, max_tokens, lambda k: parts[k], lambda k: wvecs[k],
+                                 None, None, H, True)
+        cx, cw = res[s]
+        assert np.array_equal(bf16_bits(cx), bf16_bits(ox)), s
+        assert torch.equal(cw.cpu(), ow) and torch.equal(cw.cpu(), ws[s]), s
+    for b in bufs:
+        b.destroy()

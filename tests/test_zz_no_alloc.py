@@ -2,13 +2,16 @@
 (its layout scratch is a device array inside the library).  Called through the C ABI and compared,
 bit for bit, with what ep_dispatch_launch + ep_dispatch_epilogue_launch of an ordinary buffer produce
 on the same inputs: two calls in a row, the second with a smaller input, so leftovers of the first in
-the shared scratch would show."""
+the shared scratch would show.  The first shape is also compared with the CPU oracle, and the second call
+must leave the device's free memory where it was."""
 import ctypes
 
+import numpy as np
 import pytest
 import torch
 
-from helpers import make_routing, make_tokens
+from helpers import bf16_bits, make_routing, make_tokens
+from oracle import ep_oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -54,7 +57,27 @@ def _static_dispatch(C, x, topk, w, E, A, fused):
     e.cached_mode, e.do_zero_padding, e.fused_fp8_quant, e.recv_sf_layout = 0, 1, int(fused), 0
     e.stream = a.stream
     C._check(C._ep_dispatch_static(ctypes.byref(a), ctypes.byref(e)))
+    out['_args'] = (a, e)          # (the descriptors hold raw pointers into `out` and the inputs: the caller keeps both)
     return out
+
+
+def _compare_with_oracle(out, x, topk, w, E, A, fused):
+    """The allocation-free path against the CPU oracle itself (not only against the buffer path)."""
+    T = x.size(0)
+    lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, T)
+    n_recv, upto = lay['num_recv_tokens'], lay['num_expanded_tokens']
+    assert np.array_equal(out['psum_expert'].cpu().numpy(), lay['psum_num_recv_tokens_per_expert'])
+    assert np.array_equal(out['dst_slot'].cpu().numpy(), lay['dst_buffer_slot_idx'])
+    assert np.array_equal(out['meta'][:n_recv].cpu().numpy(), lay['recv_src_metadata'])
+    if fused:
+        q, s = O.quantise(x)
+        ex, es, ew = O.rank_share_dispatch(q.numpy(), s.numpy().view(np.uint32), w.numpy(), lay)
+        assert np.array_equal(out['recv_x'][:upto].view(torch.uint8).cpu().numpy(), ex[:upto])
+        assert np.array_equal(out['recv_sf'][:upto].cpu().numpy().view(np.uint32), es[:upto])
+    else:
+        ex, _, ew = O.rank_share_dispatch(bf16_bits(x).view(np.int16), None, w.numpy(), lay)
+        assert np.array_equal(bf16_bits(out['recv_x'][:upto]).view(np.int16), ex[:upto])
+    assert np.array_equal(out['recv_w'][:upto].cpu().numpy().view(np.uint32), ew[:upto].view(np.uint32))
 
 
 def _buffer_dispatch(de, x, topk, w, E, A, fused):
@@ -96,19 +119,31 @@ def test_static_dispatch_matches_the_buffer_path_twice(fused):
     E, K, A, H = 32, 4, 16, 512
     for T, seed in ((700, 1), (130, 2)):                  # the second call is smaller: the scratch keeps the first's contents
         x = make_tokens(T, H, seed=seed, outliers=True).to(DEV)
-        topk, w = make_routing(T, E, K, seed=seed, masked=0.15)
-        topk, w = topk.to(DEV), w.to(DEV)
+        topk_cpu, w_cpu = make_routing(T, E, K, seed=seed, masked=0.15)
+        topk, w = topk_cpu.to(DEV), w_cpu.to(DEV)
         out = _static_dispatch(C, x, topk, w, E, A, fused)
         torch.cuda.synchronize()
+        if T == 700:
+            _compare_with_oracle(out, x.cpu(), topk_cpu, w_cpu, E, A, fused)
         ref = _buffer_dispatch(de, x, topk, w, E, A, fused)
         _compare(out, ref, fused, A)
+    # the entry point exists for callers that cannot allocate: a further call (every tensor it needs already
+    # exists) leaves the device's free memory untouched
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    a, e = out['_args']
+    C._check(C._ep_dispatch_static(ctypes.byref(a), ctypes.byref(e)))
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    _compare(out, ref, fused, A)
 
 
 def test_static_dispatch_rejects_what_does_not_fit():
     import deep_ep as de
     C = de._C
     C.init_jit()
-    T, H, E, K, A = 400000, 128, 8, 2, 1                 # slot map 3.2 MB + receive order 1.6 MB > 4 MiB
+    T, H, E, K, A = 400000, 128, 8, 2, 1                 # slot map 3.2 MB + token -> row map 1.6 MB > 4 MiB
+    assert C._ep_static_bytes(T, K, E) > C._ep_static_capacity() >= C._ep_static_bytes(700, 4, 32)
     x = torch.zeros((T, H), dtype=torch.bfloat16, device=DEV)
     topk = torch.zeros((T, K), dtype=torch.int64, device=DEV)
     with pytest.raises(C.EPException, match='exceeds the library\'s static scratch'):
