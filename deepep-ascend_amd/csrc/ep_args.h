@@ -175,6 +175,16 @@ struct EpCombineArgs {
     int whole_rows;               // owner-side reduce: a task is a whole row (num_parts == 1), not a 1024-channel part
 };
 
+// Caller-side quantiser: rows of BF16 -> rows of e4m3fn bytes + one fp32 scale per row and 128 channels.
+struct EpQuantArgs {
+    const void* x;                // [num_rows, hidden] BF16
+    void* q;                      // [num_rows, hidden] e4m3fn out
+    float* sf;                    // [num_rows, ceil(hidden / 128)] out
+    int num_rows, hidden;
+    int num_parts;                // 512-channel parts per row; a wave task is (row, part)
+    int hw_convert;               // 1: v_cvt_pk_fp8_f32, 0: integer conversion
+};
+
 // Hardware vs integer e4m3fn conversion over fp32 bit patterns [first, first+count).
 struct EpFp8TestArgs {
     unsigned long long first, count;

@@ -10,6 +10,7 @@
 //   ep_scatter_copy / ep_scatter_quant                     token (or receive-stream row) -> its expanded slots
 //   ep_scatter_copy_pack / ep_scatter_quant_pack           token -> one packed row per destination partition
 //   ep_sf_transpose                                        scale rows -> scale columns
+//   ep_quant_rows                                          the quantiser alone (rows in place)
 //   ep_combine_k<K> / ep_combine_generic                   K-way gather + fp32 reduce back to token order
 //   ep_combine_partial_* / ep_combine_final_*              the same reduce in its owner-side and token-side halves
 //   ep_fp8_selftest                                        hardware vs integer e4m3fn conversion
@@ -912,6 +913,38 @@ extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_pa
 }
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_scatter_quant_sw_pack(EpScatterArgs a) {
     scatter_quant_body<false, true>(a);
+}
+
+// The quantiser alone (deep_ep/utils/math.py:30-38, what a caller runs before a dispatch of pre-quantised rows):
+// the arithmetic of the fused kernel above, rows written in place of being scattered.
+template <bool HW>
+__device__ __forceinline__ void quant_rows_body(const EpQuantArgs& a) {
+    const int lane = lane_id();
+    const int task = blockIdx.x * EP_ROWS_PER_BLOCK + wave_id();
+    const int t = task / a.num_parts, part = task - t * a.num_parts;
+    if (t >= a.num_rows) return;
+    const int nvec = a.hidden >> 3;
+    const int v = part * WAVE + lane;
+    const bool live = v < nvec;
+    u32x4 d = {0u, 0u, 0u, 0u};
+    if (live) d = __builtin_nontemporal_load((const u32x4*)((const char*)a.x + (int64_t)t * a.hidden * 2) + v);
+    float f[8] = {bf16_lo(d.x), bf16_hi(d.x), bf16_lo(d.y), bf16_hi(d.y),
+                  bf16_lo(d.z), bf16_hi(d.z), bf16_lo(d.w), bf16_hi(d.w)};
+    unsigned mbits = 0u;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) mbits = max(mbits, __float_as_uint(f[q]) & 0x7fffffffu);
+    const float m = __uint_as_float(row16_umax(mbits));
+    const float amax = m < 1e-4f ? 1e-4f : m;
+    const float inv = (1.0f / amax) * 448.0f;
+    u32x2 q8 = quant8<HW>(f, inv);
+    if (amax != amax) q8 = u32x2{0x7f7f7f7fu, 0x7f7f7f7fu};
+    if (!live) return;
+    ((u32x2*)((char*)a.q + (int64_t)t * a.hidden))[v] = q8;
+    if ((lane & 15) == 0) a.sf[(int64_t)t * ((a.hidden + 127) >> 7) + (v >> 4)] = amax / 448.0f;
+}
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_quant_rows(EpQuantArgs a) {
+    if (a.hw_convert) quant_rows_body<true>(a);
+    else quant_rows_body<false>(a);
 }
 
 // Column-major scales (use_tma_aligned_col_major_sf): the copy kernels write scale rows, this

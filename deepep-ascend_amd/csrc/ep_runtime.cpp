@@ -115,7 +115,7 @@ struct Kernels {
     hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw, sf_transpose;
     hipFunction_t scatter_copy_pack, scatter_quant_pack, scatter_quant_sw_pack;
     hipFunction_t combine[3][5];     // [mode][generic, k2, k4, k6, k8]
-    hipFunction_t fp8_selftest;
+    hipFunction_t fp8_selftest, quant_rows;
     int device = -1;
 };
 
@@ -191,6 +191,7 @@ void load_kernels(const char* dir) {
         for (int k = 0; k < 5; ++k)
             get(g_k.combine[mode][k], (std::string("ep_combine") + modes[mode] + ks[k]).c_str());
     get(g_k.fp8_selftest, "ep_fp8_selftest");
+    get(g_k.quant_rows, "ep_quant_rows");
     g_k.module = m;
 }
 
@@ -395,6 +396,33 @@ int ep_fp8_selftest(uint64_t first, uint64_t count, float limit, uint64_t out[2]
         HIP_CHECK(hipFree(dev));
         out[0] = res[0];
         out[1] = res[1];
+    });
+}
+
+int ep_per_token_cast_to_fp8(const ep_tensor_t* px, const ep_tensor_t* pq, const ep_tensor_t* psf, void* stream) {
+    return guarded([&] {
+        load_kernels(nullptr);
+        EP_HOST_ASSERT(px != nullptr and pq != nullptr and psf != nullptr);
+        const ep_tensor_t &x = *px, &q = *pq, &sf = *psf;
+        EP_HOST_ASSERT(present(x) and x.ndim == 2 and x.dtype == EP_DTYPE_BF16 and contiguous(x));
+        const int64_t rows = x.size[0], hidden = x.size[1];
+        EP_HOST_ASSERT(hidden > 0 and hidden % 8 == 0 and hidden <= 16384);
+        EP_HOST_ASSERT(present(q) and q.ndim == 2 and q.size[0] == rows and q.size[1] == hidden and contiguous(q));
+        EP_HOST_ASSERT(q.dtype == EP_DTYPE_FP8_E4M3 or q.dtype == EP_DTYPE_U8);
+        EP_HOST_ASSERT(present(sf) and sf.ndim == 2 and sf.size[0] == rows and sf.size[1] == ceil_div(hidden, 128));
+        EP_HOST_ASSERT(sf.dtype == EP_DTYPE_F32 and contiguous(sf));
+        EP_HOST_ASSERT(((uintptr_t)x.data & 15) == 0 and ((uintptr_t)q.data & 7) == 0);
+        EpQuantArgs qa{};
+        qa.x = x.data;
+        qa.q = q.data;
+        qa.sf = (float*)sf.data;
+        qa.num_rows = (int)rows;
+        qa.hidden = (int)hidden;
+        qa.num_parts = (int)ceil_div(hidden, 512);
+        qa.hw_convert = g_fp8_hw ? 1 : 0;
+        const int64_t blocks = ceil_div(rows * qa.num_parts, EP_ROWS_PER_BLOCK);
+        EP_HOST_ASSERT(rows <= INT32_MAX and blocks <= INT32_MAX);
+        if (blocks > 0) launch(g_k.quant_rows, (unsigned)blocks, EP_ROW_THREADS, 0, stream, qa);
     });
 }
 

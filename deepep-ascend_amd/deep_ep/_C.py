@@ -95,6 +95,8 @@ _ep_combine_size = _sig('ep_get_combine_buffer_size', ctypes.c_int64, *([ctypes.
 _ep_host_cvt = _sig('ep_host_f32_to_e4m3fn', None, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64)
 _ep_selftest = _sig('ep_fp8_selftest', ctypes.c_int, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float,
                     ctypes.POINTER(ctypes.c_uint64))
+_ep_quantise = _sig('ep_per_token_cast_to_fp8', ctypes.c_int, ctypes.POINTER(_Tensor), ctypes.POINTER(_Tensor),
+                   ctypes.POINTER(_Tensor), ctypes.c_void_p)
 _ep_set_hw = _sig('ep_set_fp8_hw_convert', None, ctypes.c_int)
 _ep_create = _sig('ep_buffer_create', ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64,
                   ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p))
@@ -243,6 +245,19 @@ def fp8_selftest(first: int, count: int, limit: float) -> Tuple[int, int]:
     out = (ctypes.c_uint64 * 2)()
     _check(_ep_selftest(first, count, limit, out))
     return int(out[0]), int(out[1])
+
+
+def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The caller-side quantiser on the GPU (`x` a contiguous bfloat16 CUDA tensor `[T, H]`, H a multiple of 8):
+    the library's own kernel, whose bytes are those of the fused dispatch and of the formula evaluated by torch
+    on the CPU."""
+    init_jit()
+    rows, cols = x.shape
+    q = torch.empty((rows, cols), dtype=torch.float8_e4m3fn, device=x.device)
+    sf = torch.empty((rows, (cols + 127) // 128), dtype=torch.float32, device=x.device)
+    dx, dq, dsf = _desc(x), _desc(q), _desc(sf)
+    _check(_ep_quantise(ctypes.byref(dx), ctypes.byref(dq), ctypes.byref(dsf), _stream()))
+    return q, sf
 
 
 def set_fp8_hw_convert(enable: bool) -> None:

@@ -223,7 +223,9 @@ class EPBuffer(BufferBase):
                 runs the copy epilogue and returns `(recv_x, None, recv_topk_weights, handle)`.
             fused_fp8_quant (extension): `x` is bfloat16 and is quantised to e4m3fn with one fp32
                 scale per token and 128 channels on the way; returns `(recv_x_fp8, recv_sf_fp32)`
-                whose bytes equal `per_token_cast_to_fp8(x)` dispatched verbatim.
+                whose bytes equal `deep_ep.utils.math.per_token_cast_to_fp8(x)` dispatched verbatim, for
+                `x` on the GPU (the library's quantiser kernel) and on the CPU (torch's evaluation of
+                the reference formula) alike.
 
         Returns `(recv_x or (recv_x, recv_sf), None, recv_topk_weights, handle, event)`, or the
         `EventOverlap` alone when `defer_epilogue`.

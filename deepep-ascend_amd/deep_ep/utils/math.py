@@ -42,9 +42,17 @@ def count_bytes(*tensors) -> int:
 def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Caller-side quantiser (reference: deep_ep/utils/math.py:30-38): per token and per group of
     128 channels, scale = max(|x|, 1e-4) / 448 in fp32 and payload = e4m3fn(x * (448 / amax)).
-    `EPBuffer.dispatch(..., fused_fp8_quant=True)` computes the same bytes inside the dispatch."""
+
+    A contiguous bfloat16 tensor on the GPU (hidden a multiple of 8) is quantised by the library's own
+    kernel: its bytes are those `EPBuffer.dispatch(..., fused_fp8_quant=True)` writes into the slots and
+    those the formula below gives on CPU tensors.  Anything else goes through the torch formula on the
+    tensor's own device; on the GPU torch evaluates `448 / amax` with a different rounding than on the
+    CPU, so payload bytes of such inputs can differ in the last bit from the CPU's and the library's."""
     assert x.dim() == 2
     rows, cols = x.shape
+    if x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and cols % 8 == 0 and 0 < cols <= 16384:
+        from .. import _C
+        return _C.per_token_cast_to_fp8(x)
     padded = align(cols, SF_GROUP)
     groups = torch.nn.functional.pad(x, (0, padded - cols)).view(rows, padded // SF_GROUP, SF_GROUP)
     amax = groups.abs().float().amax(dim=2).clamp(1e-4)

@@ -79,6 +79,12 @@ int ep_fp8_selftest(uint64_t first, uint64_t count, float limit, uint64_t out[2]
 /* 1: hardware v_cvt_pk_fp8_f32 (default), 0: integer conversion. */
 void ep_set_fp8_hw_convert(int enable);
 
+/* The caller-side quantiser per_token_cast_to_fp8 (deep_ep/utils/math.py:30-38) on the device: x [T,H] BF16
+ * (H a multiple of 8) -> q [T,H] e4m3fn bytes and sf [T, ceil(H/128)] fp32 with, per token and per group of 128
+ * channels, sf = max(|x|, 1e-4) / 448 and q = e4m3fn(x * (448 / amax)), bit for bit what torch computes for that
+ * formula on the CPU, and what ep_dispatch_epilogue_launch with fused_fp8_quant writes into the slots. */
+int ep_per_token_cast_to_fp8(const ep_tensor_t* x, const ep_tensor_t* q, const ep_tensor_t* sf, void* stream);
+
 /* ---- buffer ---------------------------------------------------------------------------------- */
 
 /* One hipMalloc'd, zero-filled arena = workspace || buffer (num_bytes) || lb storage

@@ -273,3 +273,35 @@ def _ep32_node_checks(bufs, R, T, H, E, K, A, El):
         n_sel = (topks[r] >= 0).sum(dim=1, keepdim=True).to(torch.float32)
         assert torch.equal(cx.float(), z.float() * n_sel), r      # small integers: every sum and rounding is exact
         assert torch.equal(cw, wts[r])
+
+
+def test_65536_tokens_reach_the_scanned_layout_by_size():
+    """Four times the headline's tokens: 512 layout workgroups (beyond what the slot assignment folds itself, so the
+    scan kernel runs without any tuning knob being touched), 3.7 million wave tasks in the copy kernel.  Layout
+    against the oracle; payload, scales and padding through the layout's own properties; combine through a round
+    trip: the rows of a token are copies of it, so their sum is top-k times the token (exact in BF16 at top-4)."""
+    T, H, E, K, A = 65536, 2048, 256, 4, 128
+    x = make_tokens(T, H, seed=4, outliers=True)
+    topk, w = make_routing(T, E, K, seed=4)
+    lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, T)
+    buf = _buffer(T, H, K)                        # sized for BF16 rows: the FP8 dispatch fits as well
+    xg, tg, wg = x.to(DEV), topk.to(DEV), w.to(DEV)
+    (rx, rsf), _, rw, handle, _ = buf.dispatch(xg, topk_idx=tg, topk_weights=wg, num_experts=E, expert_alignment=A,
+                                               do_expand=True, do_zero_padding=True, fused_fp8_quant=True)
+    torch.cuda.synchronize()
+    assert handle.num_expanded_tokens == lay['num_expanded_tokens'] == rx.size(0)
+    assert np.array_equal(handle.recv_src_metadata.cpu().numpy(), lay['recv_src_metadata'])
+    assert np.array_equal(handle.psum_num_recv_tokens_per_expert.cpu().numpy(), lay['psum_num_recv_tokens_per_expert'])
+    assert np.array_equal(handle.dst_buffer_slot_idx.cpu().numpy(), lay['dst_buffer_slot_idx'])
+    q, s = O.quantise(x)
+    _check_layout_properties(handle, tg, E, A, rx.view(torch.uint8), q.to(DEV))
+    _check_layout_properties(handle, tg, E, A, rsf.view(torch.int32), s.view(torch.int32).to(DEV))
+    # BF16 round trip: dispatch the rows verbatim, combine the copies
+    rb, _, rwb, hb, _ = buf.dispatch(xg, topk_idx=tg, topk_weights=wg, num_experts=E, expert_alignment=A,
+                                     do_expand=True, do_zero_padding=True)
+    assert torch.equal(hb.recv_src_metadata, handle.recv_src_metadata)
+    cx, cw, _ = buf.combine(rb, hb, topk_weights=rwb)
+    torch.cuda.synchronize()
+    assert torch.equal(cx, xg * K)
+    assert torch.equal(cw, wg)
+    buf.destroy()

@@ -138,12 +138,15 @@ def test_fp8_dispatch_fused_and_prequantised(T, H, E, K, A, masked, zipf):
         de._C.set_fp8_hw_convert(True)
     assert torch.equal(rx2.view(torch.uint8), rx.view(torch.uint8)) and torch.equal(rsf2, rsf)
 
-    # drop-in form: caller-side quantiser, scale packs viewed as int16, row- and column-major
-    # (quantised on the CPU: torch's GPU division by a scalar rounds differently from its CPU one)
+    # drop-in form: caller-side quantiser, scale packs viewed as int16, row- and column-major.  The helper gives
+    # the oracle's bytes for a CPU tensor (torch's formula) and for a GPU tensor (the library's kernel) alike
     xq, xs = de.utils.math.per_token_cast_to_fp8(x)
     assert np.array_equal(xq.view(torch.uint8).numpy(), q.numpy())
     assert np.array_equal(xs.numpy().view(np.uint32), s.numpy().view(np.uint32))
-    xq, xs = xq.to(DEV), xs.to(DEV)
+    xq, xs = de.utils.math.per_token_cast_to_fp8(xg)
+    assert xq.is_cuda and xq.dtype == torch.float8_e4m3fn and xs.dtype == torch.float32
+    assert np.array_equal(xq.view(torch.uint8).cpu().numpy(), q.numpy())
+    assert np.array_equal(xs.cpu().numpy().view(np.uint32), s.numpy().view(np.uint32))
     sf16 = xs.view(torch.int16)
     P = sf16.size(1)
     es16 = es.view(np.int16).reshape(es.shape[0], -1)
