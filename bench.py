@@ -28,7 +28,12 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch come from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of a workload
 # (lines "traffic_bytes <kernel> <bytes>"), and only while that summary was taken from the kernel sources
 # that are being run (line "kernel_source_sha256 <hash>"); otherwise the field is null.
-TRAFFIC_PROFILES = {'c3_headline': 'headline_dispatch_combine_hbm_traffic.txt'}
+TRAFFIC_PROFILES = {'c3_headline': 'headline_dispatch_combine_hbm_traffic.txt',
+                    'c3_prequantised': 'headline_prequantised_counters.txt',
+                    'c2_bf16_top8': 'c2_bf16_top8_counters.txt',
+                    'c4_decode_zipf': 'c4_decode_zipf_counters.txt',
+                    'c5_ep32_share': 'ep32_share_counters.txt',
+                    'c5_ep32_node': 'ep32_node_counters.txt'}
 KERNEL_SOURCES = ('deepep-ascend_amd/csrc/ep_kernels.hip', 'deepep-ascend_amd/csrc/ep_args.h',
                   'deepep-ascend_amd/csrc/ep_fp8.h')
 
@@ -128,17 +133,16 @@ def cpu_model():
     return 'unknown'
 
 
-def cpu_baseline(H, E, K, A, fp8, sample_tokens, budget_s=12.0, max_passes=16):
-    """The oracle on the host cores: whole passes over `sample_tokens` tokens of the same workload, repeated
-    until about `budget_s` seconds of CPU work have been spent; and the reference's own CPU-runnable case."""
+def cpu_baseline(H, E, K, A, fp8, sample_tokens, passes=5):
+    """The oracle on the host cores over `sample_tokens` tokens of the same workload: one untimed pass, then the
+    median of `passes` timed ones (dispatch + combine); and the reference's own CPU-runnable case."""
     from oracle import ep_oracle as O
     torch.set_num_threads(os.cpu_count())
     x, topk, w = make_inputs(sample_tokens, H, E, K, seed=1)
     g = torch.Generator().manual_seed(2)
     y = None
-    t_dispatch = t_combine = 0.0
-    passes = 0
-    while passes < max_passes and (passes == 0 or t_dispatch + t_combine < budget_s):
+    times = []
+    for k in range(1 + passes):
         t0 = time.perf_counter()
         lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, sample_tokens)
         if fp8:
@@ -152,18 +156,18 @@ def cpu_baseline(H, E, K, A, fp8, sample_tokens, budget_s=12.0, max_passes=16):
         t2 = time.perf_counter()
         O.combine_fast(y, torch.from_numpy(rw), lay['recv_src_metadata'], sample_tokens, K)
         t3 = time.perf_counter()
-        t_dispatch += t1 - t0
-        t_combine += t3 - t2
-        passes += 1
+        if k >= 1:
+            times.append((t1 - t0 + t3 - t2, t1 - t0, t3 - t2))
+    times.sort()
+    med, med_d, med_c = times[len(times) // 2]
     n_valid = int(lay['num_unaligned_recv_tokens_per_expert'].sum())
     n_recv = lay['num_recv_tokens']
-    nbytes = passes * (dispatch_bytes(sample_tokens, H, K, n_valid, n_recv, fp8, True) +
-                       combine_bytes(sample_tokens, H, K, n_valid, n_recv, 0, True))
-    secs = t_dispatch + t_combine
-    return {'value': round(nbytes / secs / 1e9, 3), 'unit': 'GB/s', 'cores': torch.get_num_threads(), 'kind': 'port',
-            'cpu_model': cpu_model(),
-            'sample': f'{passes} passes over {sample_tokens} tokens of the workload: dispatch {t_dispatch:.2f} s + '
-                      f'combine {t_combine:.2f} s of numpy/torch-CPU oracle (os.cpu_count()={os.cpu_count()})',
+    nbytes = dispatch_bytes(sample_tokens, H, K, n_valid, n_recv, fp8, True) + combine_bytes(sample_tokens, H, K, n_valid, n_recv, 0, True)
+    return {'value': round(nbytes / med / 1e9, 3), 'unit': 'GB/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+            'cpu_model': cpu_model(), 'passes': passes, 'median_s': round(med, 3),
+            'sample': f'1 untimed pass, then the median of {passes} passes over {sample_tokens} tokens of the workload: '
+                      f'dispatch {med_d:.2f} s + combine {med_c:.2f} s of numpy/torch-CPU oracle '
+                      f'(os.cpu_count()={os.cpu_count()})',
             'small_case': cpu_small_case()}
 
 
@@ -318,6 +322,26 @@ def bench_partitioned(args, T, H, E, K, A, R=32, rank=5):
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
     us_d = timed_us(lambda: buf.dispatch(xg, topk_idx=tg, topk_weights=wg, **kw), args.steps)
     us_c = timed_us(lambda: buf.combine(y, handle, topk_weights=rw), args.steps)
+    # the send side alone (layout + the pack kernel, the largest of this workload): a deferred dispatch enqueues
+    # exactly that; its epilogue runs outside the bracket
+    pend = []
+
+    def send_side():
+        pend.append(buf.dispatch(xg, topk_idx=tg, topk_weights=wg, async_with_compute_stream=True, defer_epilogue=True, **kw))
+
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        a.record()
+        send_side()
+        b.record()
+        pend.pop().current_stream_wait()
+    torch.cuda.synchronize()
+    us_send = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)[len(evs) // 2]
+    traffic, traffic_source = measured_traffic(args.workload)
+    roofline = {'kernel': 'ep_scatter_quant_pack', 'bound': 'hbm', 'achieved': round(b_pack / us_send / 1e3, 1),
+                'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': round(b_pack / us_send / 1e3 / HBM_PEAK_GBS, 4),
+                'traffic': traffic.get('ep_scatter_quant_pack'), 'traffic_source': traffic_source, 'us': round(us_send, 2),
+                'measured': 'events around the send side of a dispatch (layout kernels + pack kernel), median'}
     out = {'metric': 'dispatch & combine GB/s, one GPU share of EP32 (pack 32 regions + expand own; partial + final reduce)',
            'value': round((b_pack + b_expand + b_partial + b_final) / ms / 1e6, 1), 'unit': 'GB/s', 'n_gpus': 1,
            'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms, 4), 'higher_is_better': True,
@@ -325,6 +349,7 @@ def bench_partitioned(args, T, H, E, K, A, R=32, rank=5):
            'config': {'workload': args.workload, 'tokens': T, 'hidden': H, 'experts': E, 'topk': K,
                       'expert_alignment': A, 'partitions': R, 'partition_idx': rank, 'packed_rows': n_send,
                       'received_rows': n_recv, 'valid_expanded_rows': n_valid},
+           'roofline': roofline,
            'phases': {'dispatch_us': round(us_d, 2), 'dispatch_bytes': b_pack + b_expand,
                       'dispatch_gbs': round((b_pack + b_expand) / us_d / 1e3, 1),
                       'combine_us': round(us_c, 2), 'combine_bytes': b_partial + b_final,
@@ -413,6 +438,11 @@ def bench_node(args, T, H, E, K, A, R=32, rank=5):
               'final': n_send * ctok + T * H * 2 + T * K * 12}
     us = {k: sum(v) / len(v) for k, v in phases.items()}
     share_ms = node_ms / R
+    traffic, traffic_source = measured_traffic(args.workload)
+    roofline = {'kernel': f'ep_combine_partial_k{K}', 'bound': 'hbm', 'achieved': round(nbytes['partial'] / us['partial'] / 1e3, 1),
+                'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': round(nbytes['partial'] / us['partial'] / 1e3 / HBM_PEAK_GBS, 4),
+                'traffic': traffic.get(f'ep_combine_partial_k{K}'), 'traffic_source': traffic_source, 'us': round(us['partial'], 2),
+                'measured': 'events around the owner-side reduce of one partition inside the timed node steps, mean'}
     out = {'metric': 'dispatch & combine GB/s, one partition of EP32 at its real share (all 32 partitions on one GPU, '
                      'rows and partials stored straight into peer arenas)',
            'value': round(sum(nbytes.values()) / share_ms / 1e6, 1), 'unit': 'GB/s', 'n_gpus': 1, 'steps': args.steps,
@@ -422,6 +452,7 @@ def bench_node(args, T, H, E, K, A, R=32, rank=5):
                       'expert_alignment': A, 'partitions': R, 'timed_partition': rank, 'packed_rows_sent': n_send,
                       'rows_received': n_recv, 'valid_expanded_rows': n_valid, 'node_step_ms': round(node_ms, 3),
                       'ms_per_step_is': 'node step / partitions (host clock)'},
+           'roofline': roofline,
            'phases': {k: {'us': round(us[k], 1), 'bytes': nbytes[k], 'gbs': round(nbytes[k] / us[k] / 1e3, 1)}
                       for k in us}}
     for b in bufs:
