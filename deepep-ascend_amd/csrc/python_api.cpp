@@ -51,11 +51,12 @@ int dtype_code(const at::Tensor& t, bool two_byte_packs) {
 // Empty tensors have a null data pointer while the ABI reads null as "absent": they get the address of a
 // small per-device allocation instead (never dereferenced: their sizes are zero).
 void* nonnull_ptr(const at::Tensor& t) {
-    static std::vector<at::Tensor> dummy(64);
+    // (never destroyed: at process exit torch's allocator may be gone before the statics of this module)
+    static auto* dummy = new std::vector<at::Tensor>(64);
     const int dev = t.device().has_index() ? t.device().index() : 0;
     EP_PY_ASSERT(dev >= 0 && dev < 64);
-    if (!dummy[dev].defined()) dummy[dev] = at::zeros({64}, at::TensorOptions().dtype(at::kByte).device(t.device()));
-    return dummy[dev].data_ptr();
+    if (!(*dummy)[dev].defined()) (*dummy)[dev] = at::zeros({64}, at::TensorOptions().dtype(at::kByte).device(t.device()));
+    return (*dummy)[dev].data_ptr();
 }
 
 ep_tensor_t desc(const at::Tensor& t, bool two_byte_packs = false) {
@@ -83,8 +84,9 @@ ep_tensor_t desc(const OptTensor& t, bool two_byte_packs = false) {
 void* current_stream() { return (void*)c10::hip::getCurrentHIPStream().stream(); }
 
 py::object new_event() {
-    static py::object cls = py::module_::import("deep_ep._C").attr("EventHandle");
-    return cls();
+    // (never destroyed: the interpreter is finalised before the statics of this module are)
+    static auto* cls = new py::object(py::module_::import("deep_ep._C").attr("EventHandle"));
+    return (*cls)();
 }
 
 // Uninitialised device tensors straight from torch's caching allocator (what at::empty reaches through its

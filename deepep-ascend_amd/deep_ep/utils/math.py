@@ -46,8 +46,8 @@ def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     A contiguous bfloat16 tensor on the GPU (hidden a multiple of 8) is quantised by the library's own
     kernel: its bytes are those `EPBuffer.dispatch(..., fused_fp8_quant=True)` writes into the slots and
     those the formula below gives on CPU tensors.  Anything else goes through the torch formula on the
-    tensor's own device; on the GPU torch evaluates `448 / amax` with a different rounding than on the
-    CPU, so payload bytes of such inputs can differ in the last bit from the CPU's and the library's."""
+    tensor's own device; on the GPU torch evaluates `448 / amax` and `amax / 448` with a different rounding
+    than on the CPU, so bytes of such inputs can differ in the last bit from the CPU's and the library's."""
     assert x.dim() == 2
     rows, cols = x.shape
     if x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and cols % 8 == 0 and 0 < cols <= 16384:

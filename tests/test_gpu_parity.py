@@ -504,3 +504,29 @@ def test_lb_storage_aliases_arena_tail():
     torch.cuda.synchronize()
     assert (weights == 3).all()
     buf.destroy()
+
+
+@pytest.mark.parametrize('T,H', [(1, 8), (33, 136), (7, 520), (64, 7168), (5, 16384)])
+def test_gpu_quantiser_helper_matches_the_oracle(T, H):
+    """deep_ep.utils.math.per_token_cast_to_fp8 on a GPU tensor runs the library's quantiser kernel: the oracle's
+    bytes at every row length, also where the last group of 128 channels is short, with outliers and tiny rows."""
+    g = torch.Generator().manual_seed(T * 1000 + H)
+    x = torch.randn((T, H), generator=g)
+    x[torch.rand((T, H), generator=g) < 0.01] *= 300
+    x[0] *= 1e-6                                     # a row under the 1e-4 clamp
+    x = x.to(torch.bfloat16)
+    de = _deep_ep()
+    q, s = O.quantise(x)
+    xq, xs = de.utils.math.per_token_cast_to_fp8(x.to(DEV))
+    torch.cuda.synchronize()
+    assert xq.shape == (T, H) and xs.shape == (T, (H + 127) // 128)
+    assert np.array_equal(xq.view(torch.uint8).cpu().numpy(), q.numpy())
+    assert np.array_equal(xs.cpu().numpy().view(np.uint32), s.numpy().view(np.uint32))
+    # a non-contiguous view goes through the torch formula on the tensor's own device (torch's GPU divisions round
+    # differently from its CPU ones, so no bytes are compared): it still has to be a faithful quantisation
+    wide = torch.randn((T, 2 * H), generator=g).to(torch.bfloat16).to(DEV)
+    vq, vs = de.utils.math.per_token_cast_to_fp8(wide[:, :H])
+    assert vq.shape == (T, H) and vs.shape == (T, (H + 127) // 128)
+    back = de.utils.math.per_token_cast_back(vq, vs).float()
+    ref = wide[:, :H].float()
+    assert ((back - ref).abs() <= 0.07 * ref.abs().amax(dim=1, keepdim=True) + 1e-6).all()
