@@ -220,6 +220,15 @@ def calibrate_write(ep_calib, timed, n, cargs, T, H, K, n_valid, n_recv, pad_byt
     for unit in (4, 16, 256):                                         # 16 KiB, 64 KiB, 1 MiB
         entry(f'ep_calib_fill_shuffled_{unit * 4}KiB', med(timed(lambda: ep_calib.fill(area, shuffled=unit), n)),
               pow2_bytes, f'runs of {unit} chunks ({unit * 4} KiB) kept together, the runs scrambled')
+    for modulus in (8, 32):
+        entry(f'ep_calib_fill_affine_mod{modulus}', med(timed(lambda: ep_calib.fill_affine(area, modulus), n)), pow2_bytes,
+              f'scrambled 4 KiB chunks again, but any {modulus} consecutive workgroups write chunks with {modulus} different '
+              f'indices modulo {modulus}' + (' (every XCD keeps the chunks address order gives it)' if modulus == 8 else
+                                            ' (concurrent writes spread evenly over 32 consecutive 4 KiB blocks: the interleave of the memory)'))
+    for nf in (8, 64):
+        frows = pow2_bytes // 4096 // nf
+        entry(f'ep_calib_fronts_{nf}x4KiB', med(timed(lambda: ep_calib.fronts(area, nf, frows, 4096, frows * 4096), n)), nf * frows * 4096,
+              f'{nf} regions filling up in lock step, a 4 KiB row per workgroup')
     rows = min(448, area.numel() // (256 * H))
     entry('ep_calib_fronts_256', med(timed(lambda: ep_calib.fronts(area, 256, rows, H, rows * H), n)), 256 * rows * H,
           f'256 regions filling up in lock step, one {H}-byte row per workgroup (what a gather-formulated dispatch writes)')

@@ -68,7 +68,7 @@ const char* const kVariantKernels[kNumVariants] = {
 
 struct Kernels {
     hipModule_t module = nullptr;
-    hipFunction_t fill, fill_shuffled, fronts, mixed;
+    hipFunction_t fill, fill_shuffled, fill_affine, fronts, mixed;
     hipFunction_t variant[kNumVariants];
     int device = -1;
 };
@@ -96,6 +96,7 @@ void load_kernels(const char* dir) {
     auto get = [&](hipFunction_t& fn, const char* name) { HIP_CHECK(hipModuleGetFunction(&fn, m, name)); };
     get(g_k.fill, "ep_calib_fill");
     get(g_k.fill_shuffled, "ep_calib_fill_shuffled");
+    get(g_k.fill_affine, "ep_calib_fill_affine");
     get(g_k.fronts, "ep_calib_fronts");
     get(g_k.mixed, "ep_calib_mixed");
     for (int i = 0; i < kNumVariants; ++i) get(g_k.variant[i], kVariantKernels[i]);
@@ -135,6 +136,20 @@ int ep_calib_fill(void* dst, int64_t num_bytes, int shuffled, unsigned value, vo
         CALIB_ASSERT(not shuffled or ((chunks & (chunks - 1)) == 0 and (unsigned)shuffled <= chunks));     // powers of two
         EpCalibFillArgs a = {dst, chunks, value, (unsigned)std::max(1, shuffled), 0u};
         launch(shuffled ? g_k.fill_shuffled : g_k.fill, chunks, 256, stream, a);
+    });
+}
+
+int ep_calib_fill_affine(void* dst, int64_t num_bytes, int modulus, int shift, unsigned value, void* stream) {
+    return guarded([&] {
+        load_kernels(nullptr);
+        check_device();
+        CALIB_ASSERT(dst != nullptr and ((uintptr_t)dst & 15) == 0);
+        CALIB_ASSERT(num_bytes > 0 and num_bytes % 4096 == 0 and num_bytes / 4096 <= INT32_MAX);
+        const unsigned chunks = (unsigned)(num_bytes / 4096);
+        CALIB_ASSERT(modulus > 0 and (modulus & (modulus - 1)) == 0 and (chunks & (chunks - 1)) == 0 and (unsigned)modulus <= chunks);
+        CALIB_ASSERT(shift >= 0);
+        EpCalibFillArgs a = {dst, chunks, value, (unsigned)modulus, (unsigned)shift};
+        launch(g_k.fill_affine, chunks, 256, stream, a);
     });
 }
 

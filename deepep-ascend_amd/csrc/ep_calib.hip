@@ -32,6 +32,19 @@ extern "C" __global__ __launch_bounds__(256) void ep_calib_fill_shuffled(EpCalib
     __builtin_nontemporal_store(v, p);
 }
 
+// Scrambled order that keeps every chunk on the XCD address order would give it: workgroup b writes chunk
+// scramble(b / unit_chunks) * unit_chunks + (b + shift) % unit_chunks, so that chunk index and workgroup index agree modulo
+// unit_chunks up to the shift (consecutive workgroups go to consecutive XCDs: with unit_chunks a multiple of 8 and
+// shift 0 an XCD writes the chunks it would write in address order, only at other times).
+extern "C" __global__ __launch_bounds__(256) void ep_calib_fill_affine(EpCalibFillArgs a) {
+    const unsigned unit = blockIdx.x / a.unit_chunks, in_unit = (blockIdx.x + a.pad) % a.unit_chunks;
+    const unsigned num_units = a.num_chunks / a.unit_chunks;
+    const unsigned chunk = ((unit * 0x9E3779B1u) & (num_units - 1u)) * a.unit_chunks + in_unit;
+    u32x4* p = (u32x4*)a.dst + (int64_t)chunk * 256 + threadIdx.x;
+    const u32x4 v = {a.value, a.value, a.value, a.value};
+    __builtin_nontemporal_store(v, p);
+}
+
 // num_fronts regions filling up row by row at the same pace (what the expert regions of a gather-formulated
 // dispatch look like to the memory): workgroup b writes row b / num_fronts of front b % num_fronts, one
 // 16-byte store per thread (row_bytes / 16 threads).

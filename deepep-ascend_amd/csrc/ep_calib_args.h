@@ -11,7 +11,7 @@ struct EpCalibFillArgs {
     unsigned num_chunks;
     unsigned value;
     unsigned unit_chunks;         // scrambled order: consecutive chunks that stay together (a power of two)
-    unsigned pad;
+    unsigned pad;                 // ep_calib_fill_affine: shift of the chunk inside its unit
 };
 
 // num_fronts fronts of rows: row n of front f starts at dst + f * front_pitch_bytes + n * row_bytes.

@@ -37,6 +37,7 @@ _init = _sig('ep_calib_init', ctypes.c_char_p)
 _last_error = _lib.ep_calib_last_error
 _last_error.restype = ctypes.c_char_p
 _fill = _sig('ep_calib_fill', ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p)
+_fill_affine = _sig('ep_calib_fill_affine', ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p)
 _fronts = _sig('ep_calib_fronts', ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_uint,
                ctypes.c_void_p)
 _mixed = _sig('ep_calib_mixed', ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_uint,
@@ -65,6 +66,12 @@ def fill(dst: torch.Tensor, shuffled: int = 0, value: int = 0) -> None:
     """Writes the whole of `dst` (a multiple of 4 KiB), one chunk per workgroup: in address order, or with runs
     of `shuffled` chunks in a scrambled order (powers of two)."""
     _check(_fill(dst.data_ptr(), dst.numel() * dst.element_size(), int(shuffled), value, _stream()))
+
+
+def fill_affine(dst: torch.Tensor, modulus: int, shift: int = 0, value: int = 0) -> None:
+    """Writes the whole of `dst` in a scrambled order in which workgroup b writes a chunk with index = b + shift
+    modulo `modulus`: every chunk comes from the XCD that is `shift` places after the one address order gives it."""
+    _check(_fill_affine(dst.data_ptr(), dst.numel() * dst.element_size(), modulus, shift, value, _stream()))
 
 
 def fronts(dst: torch.Tensor, num_fronts: int, rows_per_front: int, row_bytes: int, front_pitch_bytes: int) -> None:

@@ -24,6 +24,12 @@ const char* ep_calib_last_error(void);
  * the runs in a scrambled order (shuffled and the chunk count powers of two). */
 int ep_calib_fill(void* dst, int64_t num_bytes, int shuffled, unsigned value, void* stream);
 
+/* The chunks in a scrambled order again, but workgroup b writes a chunk whose index equals b + shift modulo
+ * `modulus` (a power of two, as the chunk count): consecutive workgroups go to consecutive XCDs, so with a modulus
+ * that is a multiple of 8 and shift 0 every XCD writes exactly the chunks it writes in address order, only at
+ * other times; a shift moves every chunk to another XCD. */
+int ep_calib_fill_affine(void* dst, int64_t num_bytes, int modulus, int shift, unsigned value, void* stream);
+
 /* num_fronts regions, front_pitch_bytes apart, filling up row by row in lock step: workgroup b writes row
  * b / num_fronts of front b % num_fronts (row_bytes a multiple of 16, at most 16384). */
 int ep_calib_fronts(void* dst, int num_fronts, int rows_per_front, int row_bytes, int64_t front_pitch_bytes,

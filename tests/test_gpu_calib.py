@@ -90,6 +90,10 @@ def test_calibration_fills_write_every_byte():
     area.zero_()
     ep_calib.fill(area, shuffled=4, value=0x02020202)
     assert int(area.sum()) == 2 * area.numel()
+    for modulus, shift in ((8, 0), (32, 5)):
+        area.zero_()
+        ep_calib.fill_affine(area, modulus, shift, value=0x03030303)
+        assert int(area.sum()) == 3 * area.numel()
     area.zero_()
     ep_calib.fronts(area, 8, 16, 7168, 16 * 7168 + 4096)
     torch.cuda.synchronize()
