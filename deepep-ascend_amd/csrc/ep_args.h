@@ -52,10 +52,11 @@ struct EpLayoutArgs {
     int scan_mode;                // EP_LAYOUT_*: where ep_layout_assign finds the other blocks' counts
     // scratch (device)
     int* blk_cnt;                 // [num_blocks, cnt_stride]  per workgroup: entries per local expert (columns [0, El)),
-                                  //   masters per partition (columns [El, El + R)), zeros up to the stride; after
-                                  //   ep_layout_scan the exclusive prefix over the workgroups instead
+                                  //   masters per partition (columns [El, El + R)), zeros up to the stride: 16-bit counts
+                                  //   (EP_LAYOUT_FOLDED), or ints that ep_layout_scan replaces by the exclusive prefix
+                                  //   over the workgroups (EP_LAYOUT_SCANNED)
     int* col_total;               // [cnt_stride]  column totals (written by ep_layout_scan)
-    int cnt_stride;               // El + R rounded up to a multiple of 4 ints
+    int cnt_stride;               // El + R rounded up to a multiple of 8 columns
     int* slot_map;                // [T, K]  expanded slot of (t, j) if its expert is local, else -1
     int* tok_row;                 // [T]  token -> its row of the receive stream (written for received tokens only)
     // handle tensors (device)

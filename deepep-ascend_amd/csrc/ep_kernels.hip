@@ -25,6 +25,7 @@
 #define WAVE 64
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 // Streaming stores of the row kernels.  The policy bits of the store instruction (sc0, sc1 = scope,
@@ -125,14 +126,15 @@ __device__ __forceinline__ int64_t recv_packed_row(const int* psum, int R, int m
 // Stages the expert ids of this workgroup's entries.  Send side: entry (t, j) of topk_idx.  Receive
 // side: entry (row, j) of the receive stream, read from the packed row; partitions play no role there.
 // num_rows: rows (tokens) the entries range over (layout_num_rows).
-__device__ __forceinline__ int layout_num_rows(const EpLayoutArgs& a, int* s_psum) {
-    return a.recv_mode ? recv_scan_sources(a, s_psum) : a.num_tokens;
+// (recv: a.recv_mode, or the constant an instance of the slot assignment was built for)
+__device__ __forceinline__ int layout_num_rows(const EpLayoutArgs& a, int* s_psum, bool recv) {
+    return recv ? recv_scan_sources(a, s_psum) : a.num_tokens;
 }
 __device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s_key, short* s_rk, const int* s_psum,
-                                                 int num_rows) {
+                                                 int num_rows, bool recv) {
     const int K = a.num_topk;
     const int n = EP_TOKENS_PER_BLOCK * K;
-    if (a.recv_mode) {
+    if (recv) {
         const int N = num_rows;
         for (int i = threadIdx.x; i < n; i += blockDim.x) {
             const int row = i / K, j = i - row * K;
@@ -174,10 +176,9 @@ __device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s
 
 // Destination partition of entry idx if it is the last slot of its token going there, else -1
 // (the "master" of common/simt.hpp:24-34).
-__device__ __forceinline__ int master_rank(const short* s_rk, int idx, int K) {
+__device__ __forceinline__ int master_rank(const short* s_rk, int idx, int j, int K) {      // j = idx % K
     const int r = s_rk[idx];
     if (r < 0) return -1;
-    const int j = idx % K;
     for (int jj = j + 1; jj < K; ++jj)
         if (s_rk[idx - j + jj] == r) return -1;
     return r;
@@ -196,21 +197,34 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(
     short* s_rk = s_key + EP_TOKENS_PER_BLOCK * K;
     int* s_psum = (int*)(s_rk + EP_TOKENS_PER_BLOCK * K);      // [R + waves]  (receive side)
     for (int i = threadIdx.x; i < E + R; i += blockDim.x) smem[i] = 0;
-    const int num_rows = layout_num_rows(a, s_psum);
+    const int num_rows = layout_num_rows(a, s_psum, a.recv_mode != 0);
     // the scan stops at the last workgroup that has rows: the ones behind it leave nothing
     if ((int)blockIdx.x > 0 && (int)blockIdx.x * EP_TOKENS_PER_BLOCK >= num_rows) return;
-    layout_load_keys(a, s_key, s_rk, s_psum, num_rows);
+    layout_load_keys(a, s_key, s_rk, s_psum, num_rows, a.recv_mode != 0);
     __syncthreads();
     const int n = EP_TOKENS_PER_BLOCK * K;
+    // (the position of an entry inside its token is carried along: a division by a run-time top-k is forty instructions)
+    int j = (int)threadIdx.x % K;
+    const int jstep = (int)blockDim.x % K;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         const int e = s_key[i];
         if (e >= 0) atomicAdd(&s_ecnt[e], 1);
-        const int mr = master_rank(s_rk, i, K);
+        const int mr = master_rank(s_rk, i, j, K);
         if (mr >= 0) atomicAdd(&s_rcnt[mr], 1);
+        j += jstep;
+        if (j >= K) j -= K;
     }
     __syncthreads();
-    // one row of the count matrix: this partition's experts, then the partitions, then zero fill
+    // one row of the count matrix: this partition's experts, then the partitions, then zero fill.  For the scan kernel
+    // the counts are ints; the slot assignment that sums the rows itself takes them as 16-bit halves (a count is at
+    // most EP_TOKENS_PER_BLOCK * EP_MAX_TOPK = 4096), eight columns a 16-byte load and two columns an add.
     const int El = a.experts_per_rank, lo = a.rank_idx * El;
+    if (a.scan_mode == EP_LAYOUT_FOLDED) {
+        unsigned* row = (unsigned*)a.blk_cnt + (int64_t)blockIdx.x * (a.cnt_stride >> 1);
+        auto count_of = [&](int i) -> unsigned { return i < El ? s_ecnt[lo + i] : (i < El + R ? s_rcnt[i - El] : 0); };
+        for (int i = threadIdx.x; i < (a.cnt_stride >> 1); i += blockDim.x) row[i] = count_of(2 * i) | count_of(2 * i + 1) << 16;
+        return;
+    }
     int* row = a.blk_cnt + (int64_t)blockIdx.x * a.cnt_stride;
     for (int i = threadIdx.x; i < a.cnt_stride; i += blockDim.x)
         row[i] = i < El ? s_ecnt[lo + i] : (i < El + R ? s_rcnt[i - El] : 0);
@@ -272,13 +286,13 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
 //   slot_map[t,j]            = expert_start[e] + number of earlier (t',j') entries with the same
 //                               local expert (lexicographic order)    -- dispatch_copy_epilogue.hpp:471-488
 //                               with the canonical order of deep_ep/buffers/ep.py:100-160
-// Block 0 also publishes the per-partition / per-expert counts and prefix sums
-// (impls/ep/dispatch.hpp:469-545) and, when asked, the host count page.
+// One workgroup (the only one, or one launched beside the ranking ones) publishes the per-partition / per-expert
+// counts and prefix sums (impls/ep/dispatch.hpp:469-545) and, when asked, the host count page.
 //
 // Where the counts of the other blocks come from (a.scan_mode):
 //   EP_LAYOUT_SCANNED  ep_layout_scan left exclusive prefixes in blk_cnt and totals in col_total
-//   EP_LAYOUT_FOLDED   ep_layout_count left plain counts in blk_cnt: every block sums the rows before it
-//                      itself (cheaper than a launch of its own up to a few hundred blocks)
+//   EP_LAYOUT_FOLDED   ep_layout_count left plain counts in blk_cnt (16-bit halves): every block sums the rows
+//                      before it itself (cheaper than a launch of its own up to a few hundred blocks)
 //   EP_LAYOUT_SINGLE   one block owns every token: nothing ran before, its own LDS counts are the totals
 // Only the local experts and the partitions need prefixes: slots of other experts are never used.
 // ------------------------------------------------------------------------------------------------
@@ -286,7 +300,10 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
 #define EP_KEY_MASTER 0x4000          // flag in a staged key: the entry is the master of its partition (ids < 2048)
 #define EP_LAYOUT_MAX_COLS_PER_THREAD ((EP_MAX_EXPERTS + EP_MAX_RANKS + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS)
 
-extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign(EpLayoutArgs a) {
+// Four instances.  FOLD: for EP_LAYOUT_FOLDED (the other modes run one without the summing code).  RECV: for the
+// receive side of a node (a.recv_mode).
+template <bool FOLD, bool RECV>
+__device__ __forceinline__ void layout_assign_body(const EpLayoutArgs& a) {
     extern __shared__ int smem[];
     const int E = a.num_experts, R = a.num_ranks, K = a.num_topk, El = a.experts_per_rank, A = a.expert_alignment;
     const int NW = EP_LAYOUT_THREADS / WAVE;
@@ -302,87 +319,113 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     const int lo = a.rank_idx * El;
     const int ncols = El + R;              // column c < El: local expert lo + c; else partition c - El
 
-    const int num_rows = layout_num_rows(a, s_psum);
-    if (b > 0 && b * EP_TOKENS_PER_BLOCK >= num_rows) return;      // nothing to rank here, nothing to publish
+    // With more than one block of tokens the launch has one workgroup more than blocks.  It ranks nothing: it sums the
+    // counts like the others and publishes the totals (handle tensors, inboxes, the host count page with its two
+    // system-scope fences), so that no ranking workgroup has that on its way.
+    const bool single = !FOLD && a.scan_mode == EP_LAYOUT_SINGLE;     // (the summing instance never runs alone)
+    const bool publisher = single || b == a.num_blocks, worker = single || b < a.num_blocks;
+    const int num_rows = layout_num_rows(a, s_psum, RECV);
+    if (!publisher && b > 0 && b * EP_TOKENS_PER_BLOCK >= num_rows) return;      // nothing to rank here
 
     // ---- counts of the workgroups before this one (kept in registers) and totals over all of them ----
     int pre[EP_LAYOUT_MAX_COLS_PER_THREAD], tot[EP_LAYOUT_MAX_COLS_PER_THREAD];
 #pragma unroll
     for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) pre[k] = tot[k] = 0;
-    if (a.scan_mode == EP_LAYOUT_SCANNED) {
+    if (!FOLD && a.scan_mode == EP_LAYOUT_SCANNED) {
 #pragma unroll
         for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
             const int c = tid + k * EP_LAYOUT_THREADS;
             if (c >= ncols) continue;
-            pre[k] = a.blk_cnt[(int64_t)b * a.cnt_stride + c];
+            if (worker) pre[k] = a.blk_cnt[(int64_t)b * a.cnt_stride + c];
             tot[k] = a.col_total[c];
         }
     }
-    // This workgroup's expert ids are asked for before the sums below and land while those wait for their rows
-    // (send side, up to four ids a thread).
+    // This workgroup's expert ids are asked for first (send side, up to four ids a thread).
     const int nkeys = EP_TOKENS_PER_BLOCK * K;
     const int64_t key_base = (int64_t)b * nkeys, key_total = (int64_t)a.num_tokens * K;
-    const bool keys_early = a.scan_mode == EP_LAYOUT_FOLDED && !a.recv_mode && nkeys <= 4 * EP_LAYOUT_THREADS && key_total > 0;
-    int64_t pk[4] = {-1, -1, -1, -1};
+    const bool folded = FOLD;
+    const bool keys_early = folded && !RECV && nkeys <= 4 * EP_LAYOUT_THREADS && key_total > 0;
+    // EP_LAYOUT_FOLDED: ep_layout_count has finished and left plain counts as 16-bit halves; the rows before this
+    // workgroup's (and all rows) are summed here.  A thread takes 8 adjacent columns (one 16-byte load a row) of every
+    // S-th row, EP_FOLD_DEPTH loads in flight, and adds them two columns an instruction: each half of the rows in flight
+    // has 16-bit sums of its own (EP_FOLD_DEPTH / 2 rows of at most 4096 stay below 2^16), widened at its end; the S
+    // partial sums of a column meet in LDS.  The rows come from memory (other XCDs wrote
+    // them) and that trip is the longest wait of the kernel: the first turn's rows are asked for here and summed only
+    // after the keys have been staged and counted per wave, which needs none of them.
+    const int W = a.cnt_stride, FG = W >> 3;
+    int* s_fpre = s_psum + R + NW;         // [W]  (EP_LAYOUT_FOLDED only)
+    int* s_ftot = s_fpre + W;              // [W]
+    const int nb = min(a.num_blocks, max(1, (num_rows + EP_TOKENS_PER_BLOCK - 1) / EP_TOKENS_PER_BLOCK));
+    const int S = FG >= EP_LAYOUT_THREADS ? 1 : EP_LAYOUT_THREADS / FG;
+    const int s0 = FG >= EP_LAYOUT_THREADS ? 0 : tid / FG;
+    const int g0 = FG >= EP_LAYOUT_THREADS ? tid : tid - s0 * FG;
+    // (rows are addressed by a 32-bit offset from the uniform base: two instructions a load)
+    const unsigned row_bytes = (unsigned)W * 2u, step = (unsigned)S * row_bytes;
+    auto fold_loads = [&](u32x4 (&v)[EP_FOLD_DEPTH], int r, int g) {
+        const unsigned off = (unsigned)r * row_bytes + 16u * g, last = (unsigned)(nb - 1) * row_bytes + 16u * g;
+        // unconditional loads (a row past the end re-reads the last one and is masked in the sums), so that all of
+        // them are in flight before the first is waited for
+#pragma unroll
+        for (int u = 0; u < EP_FOLD_DEPTH; ++u) v[u] = *(const u32x4*)((const char*)a.blk_cnt + min(off + u * step, last));
+        __builtin_amdgcn_sched_barrier(0);          // (the scheduler otherwise sums the first rows before it asks for the last)
+    };
+    auto fold_sums = [&](const u32x4 (&v)[EP_FOLD_DEPTH], int r, int (&p)[8], int (&t)[8]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            // (a short launch has no rows in the second half of a turn: its adds are skipped)
+            if (h == 1 && r + (EP_FOLD_DEPTH / 2) * S >= nb) break;
+            u16x2 ts[4], ps[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) ts[q] = ps[q] = u16x2{0, 0};
+#pragma unroll
+            for (int u = h * (EP_FOLD_DEPTH / 2); u < (h + 1) * (EP_FOLD_DEPTH / 2); ++u) {
+                const int rr = r + u * S;
+                const unsigned mt = rr < nb ? ~0u : 0u, mp = rr < b ? ~0u : 0u;      // b <= nb - 1
+                ts[0] += __builtin_bit_cast(u16x2, v[u].x & mt); ps[0] += __builtin_bit_cast(u16x2, v[u].x & mp);
+                ts[1] += __builtin_bit_cast(u16x2, v[u].y & mt); ps[1] += __builtin_bit_cast(u16x2, v[u].y & mp);
+                ts[2] += __builtin_bit_cast(u16x2, v[u].z & mt); ps[2] += __builtin_bit_cast(u16x2, v[u].z & mp);
+                ts[3] += __builtin_bit_cast(u16x2, v[u].w & mt); ps[3] += __builtin_bit_cast(u16x2, v[u].w & mp);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                t[2 * q] += (int)ts[q].x;
+                t[2 * q + 1] += (int)ts[q].y;
+                p[2 * q] += (int)ps[q].x;
+                p[2 * q + 1] += (int)ps[q].y;
+            }
+        }
+    };
+    // (Lanes are 8 columns apart: column 8 g + q lives at 8 g + ((q + g / 4) & 7), which spreads the 32 lanes of one
+    //  add over the 32 banks instead of four.)
+    auto fold_meet = [&](int g, const int (&p)[8], const int (&t)[8]) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const int at = 8 * g + ((q + (g >> 2)) & 7);
+            atomicAdd(&s_fpre[at], p[q]);
+            atomicAdd(&s_ftot[at], t[q]);
+        }
+    };
+    // (the host sends shapes with more than 8 * EP_LAYOUT_THREADS count columns to the scan kernel: one column group a thread)
+    const bool fold_mine = folded && s0 < S && g0 < FG;        // this thread sums rows
+
+    // ---- A: stage this block's keys, clear the per-wave counters (and where the sums of the rows meet) ----
+    // Every thread asks for rows and only the ones that sum look at what arrives; both ways through this phase leave
+    // the same EP_FOLD_DEPTH loads in flight.  (The compiler counts the loads in flight along every path: with the
+    // rows asked for on one path only, or under a per-thread condition, it waits for all of them at the next loop.)
+    u32x4 v_first[EP_FOLD_DEPTH];
+    auto clear_counters = [&]() {
+        for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
+        if (folded)
+            for (int i = tid; i < 2 * W; i += blockDim.x) s_fpre[i] = 0;
+    };
     if (keys_early) {
+        // ids first, rows behind them; the ids are staged while the rows are on their way
+        int64_t pk[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) pk[u] = a.topk_idx[min(key_base + tid + u * EP_LAYOUT_THREADS, key_total - 1)];
         __builtin_amdgcn_sched_barrier(0);
-    }
-    if (a.scan_mode == EP_LAYOUT_FOLDED) {
-        // ep_layout_count has finished and left plain counts: sum the rows before this workgroup's (and all
-        // rows) here.  A thread takes 4 adjacent columns (one 16-byte load a row) of every S-th row, EP_FOLD_DEPTH
-        // loads in flight (the rows come from memory: other XCDs wrote them); the S partial sums of a column
-        // meet in LDS (the per-wave counters are not in use yet).
-        const int W = a.cnt_stride, G = W >> 2;
-        int* s_fpre = s_we;                // [W]
-        int* s_ftot = s_we + W;            // [W]   (2 W <= NW * (E + R) ints)
-        for (int i = tid; i < 2 * W; i += blockDim.x) s_we[i] = 0;
-        __syncthreads();
-        const int nb = min(a.num_blocks, max(1, (num_rows + EP_TOKENS_PER_BLOCK - 1) / EP_TOKENS_PER_BLOCK));
-        const int S = G >= EP_LAYOUT_THREADS ? 1 : EP_LAYOUT_THREADS / G;
-        const int s0 = G >= EP_LAYOUT_THREADS ? 0 : tid / G;
-        if (s0 < S) {
-            for (int g = G >= EP_LAYOUT_THREADS ? tid : tid % G; g < G; g += EP_LAYOUT_THREADS) {
-                const u32x4* base = (const u32x4*)(a.blk_cnt + 4 * g);
-                const int64_t vstride = W >> 2;
-                int p0 = 0, p1 = 0, p2 = 0, p3 = 0, t0 = 0, t1 = 0, t2 = 0, t3 = 0;
-                for (int r = s0; r < nb; r += EP_FOLD_DEPTH * S) {
-                    u32x4 v[EP_FOLD_DEPTH];
-#pragma unroll
-                    for (int u = 0; u < EP_FOLD_DEPTH; ++u) {
-                        // unconditional loads (a row past the end re-reads the last one and is masked below), so
-                        // that all of them are in flight before the first is waited for
-                        v[u] = base[(int64_t)min(r + u * S, nb - 1) * vstride];
-                    }
-#pragma unroll
-                    for (int u = 0; u < EP_FOLD_DEPTH; ++u) {
-                        const int rr = r + u * S;
-                        const int mt = rr < nb ? -1 : 0, mp = rr < b ? -1 : 0;      // b <= nb - 1
-                        t0 += (int)v[u].x & mt; t1 += (int)v[u].y & mt; t2 += (int)v[u].z & mt; t3 += (int)v[u].w & mt;
-                        p0 += (int)v[u].x & mp; p1 += (int)v[u].y & mp; p2 += (int)v[u].z & mp; p3 += (int)v[u].w & mp;
-                    }
-                }
-                atomicAdd(&s_fpre[4 * g], p0); atomicAdd(&s_fpre[4 * g + 1], p1);
-                atomicAdd(&s_fpre[4 * g + 2], p2); atomicAdd(&s_fpre[4 * g + 3], p3);
-                atomicAdd(&s_ftot[4 * g], t0); atomicAdd(&s_ftot[4 * g + 1], t1);
-                atomicAdd(&s_ftot[4 * g + 2], t2); atomicAdd(&s_ftot[4 * g + 3], t3);
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
-            const int c = tid + k * EP_LAYOUT_THREADS;
-            if (c >= ncols) continue;
-            pre[k] = s_fpre[c];
-            tot[k] = s_ftot[c];
-        }
-        __syncthreads();
-    }
-
-    // ---- A: stage this block's keys, clear the per-wave counters ----
-    for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
-    if (keys_early) {
+        if (FOLD) fold_loads(v_first, s0, min(g0, FG - 1));
+        clear_counters();
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int i = tid + u * EP_LAYOUT_THREADS;
@@ -392,7 +435,9 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             s_rk[i] = (short)(e < 0 ? -1 : e / a.experts_per_rank);
         }
     } else {
-        layout_load_keys(a, s_key, s_rk, s_psum, num_rows);
+        clear_counters();
+        layout_load_keys(a, s_key, s_rk, s_psum, num_rows, RECV);
+        if (FOLD) fold_loads(v_first, s0, min(g0, FG - 1));
     }
     __syncthreads();
 
@@ -400,19 +445,48 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     const int n = EP_TOKENS_PER_BLOCK * K;
     const int rounds = (n + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS;
     const int epw = rounds * WAVE;
-    for (int rd = 0; rd < rounds; ++rd) {
+    // (token and position of this lane's entry of a round are carried along instead of divided out every round)
+    const int tok0 = (w * epw + lane) / K, pos0 = (w * epw + lane) - tok0 * K;
+    const int tok_step = WAVE / K, pos_step = WAVE - tok_step * K;
+    for (int rd = 0, pos = pos0; rd < rounds; ++rd) {
         const int idx = w * epw + rd * WAVE + lane;
         if (idx < n) {
             const int e = s_key[idx];
             if (e >= 0) atomicAdd(&s_we[w * E + e], 1);
-            const int mr = master_rank(s_rk, idx, K);
+            const int mr = master_rank(s_rk, idx, pos, K);
             if (mr >= 0) {
                 atomicAdd(&s_wr[w * R + mr], 1);
                 s_key[idx] = (short)(e | EP_KEY_MASTER);        // remembered for the ranking (only this thread reads it)
             }
         }
+        pos += pos_step;
+        if (pos >= K) pos -= K;
+    }
+
+    // ---- the rows asked for at the top: counts of the workgroups before this one, totals over all ----
+    if (fold_mine) {
+        int p[8], t[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) p[q] = t[q] = 0;
+        fold_sums(v_first, s0, p, t);
+        for (int r = s0 + EP_FOLD_DEPTH * S; r < nb; r += EP_FOLD_DEPTH * S) {
+            u32x4 v[EP_FOLD_DEPTH];
+            fold_loads(v, r, g0);
+            fold_sums(v, r, p, t);
+        }
+        fold_meet(g0, p, t);
     }
     __syncthreads();
+    if (folded) {
+#pragma unroll
+        for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
+            const int c = tid + k * EP_LAYOUT_THREADS;
+            if (c >= ncols) continue;
+            const int at = (c & ~7) | ((c + (c >> 5)) & 7);
+            pre[k] = s_fpre[at];
+            tot[k] = s_ftot[at];
+        }
+    }
 
     // ---- C: totals over all workgroups into LDS (one workgroup: its own per-wave counts are the totals) ----
 #pragma unroll
@@ -432,7 +506,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     __syncthreads();
 
     // ---- D + E: aligned exclusive scan over the local experts (totals are replaced in place by the
-    //      first slot of each expert); block 0 publishes the handle tensors and the host count page ----
+    //      first slot of each expert); the publishing workgroup writes the handle tensors and the host count page ----
     int* s_start = s_tot;
     const int per = (El + EP_LAYOUT_THREADS - 1) / EP_LAYOUT_THREADS;
     const int e0 = min(El, tid * per), e1 = min(El, e0 + per);
@@ -450,7 +524,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
         int run = wave_off + incl - mine;
         for (int e = e0; e < e1; ++e) {
             const int c = s_tot[e];
-            if (b == 0 && !a.send_only) {
+            if (publisher && !a.send_only) {
                 a.unaligned_expert[e] = c;
                 a.psum_expert[e] = run + c;
                 if (a.cumulative_stats != nullptr) atomicAdd(&a.cumulative_stats[e], c);
@@ -460,7 +534,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             run += align_up(c, A);
         }
     }
-    if (b == 0 && a.send_only) {
+    if (publisher && a.send_only) {
         // rows this partition sends to every partition, left in the receivers' inboxes: the count half of
         // the reference's cross-rank reduction (impls/ep/dispatch.hpp:469-545)
         // (a partition that is not connected to a node only has its own inbox)
@@ -468,13 +542,13 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             if (a.connected || r == a.rank_idx)
                 ((int*)(a.peer_arenas[r] + EP_WS_INBOX_OFF))[a.rank_idx] = min(s_tot[El + r], a.max_tokens);
     }
-    if (b == 0 && !a.send_only) {
+    if (publisher && !a.send_only) {
         // one partition: the receive stream is this partition's own routed tokens; several: the rows counted
         // in the inbox (csrc/buffers/ep.hpp:205-246 names the tensors)
-        const int n_recv = a.recv_mode ? num_rows : s_tot[El + a.rank_idx];
+        const int n_recv = RECV ? num_rows : s_tot[El + a.rank_idx];
         for (int r = tid; r < R; r += blockDim.x) {
-            const int upto = a.recv_mode ? s_psum[r] : n_recv;
-            const int from = a.recv_mode && r ? s_psum[r - 1] : 0;
+            const int upto = RECV ? s_psum[r] : n_recv;
+            const int from = RECV && r ? s_psum[r - 1] : 0;
             a.psum_rank[r] = upto;
             if (a.notify_host) a.host_page[EP_HOST_RANK_OFF + r] = upto - from;
         }
@@ -489,6 +563,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
             }
         }
     }
+    if (!worker) return;
     __syncthreads();
 
     // ---- F: counts -> starting slots (global base + blocks before + waves before) ----
@@ -513,7 +588,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
     const int rbits = 32 - __builtin_clz(R);
     const uint64_t lt = (1ull << lane) - 1ull;
     const int64_t total = (int64_t)num_rows * K;
-    for (int rd = 0; rd < rounds; ++rd) {
+    for (int rd = 0, tok = tok0, pos = pos0; rd < rounds; ++rd) {
         const int idx = w * epw + rd * WAVE + lane;
         const bool in = idx < n;
         const int key = in ? s_key[idx] : -1;
@@ -534,7 +609,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
         }
         const int64_t g = (int64_t)b * n + idx;
         if (in && g < total) {
-            if (a.recv_mode) {
+            if (RECV) {
                 const int64_t row = g / K;
                 if (row < a.rows_cap) a.recv_src_metadata[row * (K + 2) + (g - row * K)] = eslot;
             } else {
@@ -542,15 +617,18 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
                 a.dst_gsge_idx[g] = -1;             // every copy is local: no transport descriptors
                 if (!a.send_only) {
                     a.slot_map[g] = eslot;
-                    if (mr == a.rank_idx) a.tok_row[b * EP_TOKENS_PER_BLOCK + idx / K] = rslot;
+                    if (mr == a.rank_idx) a.tok_row[b * EP_TOKENS_PER_BLOCK + tok] = rslot;
                 }
             }
         }
         // the running counters of a wave are touched by that wave only and the LDS operations of a wave
         // complete in order: no block barrier (which would also wait for the stores above) is needed
         __builtin_amdgcn_wave_barrier();
+        tok += tok_step;
+        pos += pos_step;
+        if (pos >= K) { pos -= K; ++tok; }
     }
-    if (a.recv_mode) {
+    if (RECV) {
         // the two trailing columns of the metadata rows: source token and last local selection
         // (dispatch_copy_epilogue.hpp:514-522)
         for (int row = tid; row < EP_TOKENS_PER_BLOCK; row += blockDim.x) {
@@ -569,6 +647,11 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign
         }
     }
 }
+
+extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign(EpLayoutArgs a) { layout_assign_body<false, false>(a); }
+extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign_fold(EpLayoutArgs a) { layout_assign_body<true, false>(a); }
+extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign_recv(EpLayoutArgs a) { layout_assign_body<false, true>(a); }
+extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_assign_fold_recv(EpLayoutArgs a) { layout_assign_body<true, true>(a); }
 
 // ------------------------------------------------------------------------------------------------
 // Scatter (dispatch copy epilogue): a wave task is one column part of one row (a token, or a row of the receive stream).

@@ -111,7 +111,7 @@ int64_t combine_buffer_size(int ranks, int max_tokens, int hidden, int topk) {
 // ---- code object ------------------------------------------------------------------------------
 struct Kernels {
     hipModule_t module = nullptr;
-    hipFunction_t layout_count, layout_scan, layout_assign;
+    hipFunction_t layout_count, layout_scan, layout_assign[2][2];      // [sums the counts itself][receive side]
     hipFunction_t scatter_copy, scatter_quant, scatter_quant_sw, sf_transpose;
     hipFunction_t scatter_copy_pack, scatter_quant_pack, scatter_quant_sw_pack;
     hipFunction_t combine[3][5];     // [mode][generic, k2, k4, k6, k8]
@@ -177,7 +177,10 @@ void load_kernels(const char* dir) {
     auto get = [&](hipFunction_t& fn, const char* name) { HIP_CHECK(hipModuleGetFunction(&fn, m, name)); };
     get(g_k.layout_count, "ep_layout_count");
     get(g_k.layout_scan, "ep_layout_scan");
-    get(g_k.layout_assign, "ep_layout_assign");
+    get(g_k.layout_assign[0][0], "ep_layout_assign");
+    get(g_k.layout_assign[1][0], "ep_layout_assign_fold");
+    get(g_k.layout_assign[0][1], "ep_layout_assign_recv");
+    get(g_k.layout_assign[1][1], "ep_layout_assign_fold_recv");
     get(g_k.scatter_copy, "ep_scatter_copy");
     get(g_k.scatter_quant, "ep_scatter_quant");
     get(g_k.scatter_quant_sw, "ep_scatter_quant_sw");
@@ -273,9 +276,10 @@ unsigned layout_key_bytes(int K) { return 2u * EP_TOKENS_PER_BLOCK * K * sizeof(
 unsigned layout_count_lds(int E, int R, int K) {
     return (unsigned)(E + R + R + EP_LAYOUT_THREADS / 64) * sizeof(int) + layout_key_bytes(K);
 }
-unsigned layout_assign_lds(int E, int R, int K) {
+// (cnt_stride > 0: the assignment sums the count rows itself and needs two rows of ints where the partial sums meet)
+unsigned layout_assign_lds(int E, int R, int K, int cnt_stride) {
     const unsigned nw = EP_LAYOUT_THREADS / 64;
-    return (unsigned)(E / R + R + nw * (E + R) + nw + 1 + R + nw) * sizeof(int) + layout_key_bytes(K);
+    return (unsigned)(E / R + R + nw * (E + R) + nw + 1 + R + nw + 2 * cnt_stride) * sizeof(int) + layout_key_bytes(K);
 }
 
 // The layout pass: per-block histograms, then the slot assignment.  One block needs no histogram pass; up
@@ -283,14 +287,20 @@ unsigned layout_assign_lds(int E, int R, int K) {
 // beyond that a scan kernel turns them into prefixes first.
 void launch_layout(EpLayoutArgs& la, int num_blocks, void* stream) {
     const int E = la.num_experts, R = la.num_ranks, K = la.num_topk;
-    const unsigned smem_assign = layout_assign_lds(E, R, K);
+    // (the few shapes with more count columns than the summing instance has threads for, or whose LDS would not hold
+    //  the rows where its sums meet, take the scan kernel at any size)
+    const bool fold = num_blocks <= g_fold_max_blocks and la.cnt_stride <= 8 * EP_LAYOUT_THREADS and
+                      layout_assign_lds(E, R, K, la.cnt_stride) <= 64 * 1024;
+    la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : (fold ? EP_LAYOUT_FOLDED : EP_LAYOUT_SCANNED);
+    const unsigned smem_assign = layout_assign_lds(E, R, K, la.scan_mode == EP_LAYOUT_FOLDED ? la.cnt_stride : 0);
     EP_HOST_ASSERT(smem_assign <= 64 * 1024);
-    la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : (num_blocks <= g_fold_max_blocks ? EP_LAYOUT_FOLDED : EP_LAYOUT_SCANNED);
     if (la.scan_mode != EP_LAYOUT_SINGLE)
         launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, layout_count_lds(E, R, K), stream, la);
     if (la.scan_mode == EP_LAYOUT_SCANNED)
         launch(g_k.layout_scan, (unsigned)ceil_div(la.cnt_stride, 16), EP_SCAN_THREADS, 0, stream, la);
-    launch(g_k.layout_assign, num_blocks, EP_LAYOUT_THREADS, smem_assign, stream, la);
+    // (several blocks: one workgroup more, which publishes the totals and ranks nothing)
+    launch(g_k.layout_assign[la.scan_mode == EP_LAYOUT_FOLDED][la.recv_mode != 0],
+           (unsigned)num_blocks + (la.scan_mode == EP_LAYOUT_SINGLE ? 0u : 1u), EP_LAYOUT_THREADS, smem_assign, stream, la);
 }
 
 void write_peer_table(ep_buffer* b, const std::vector<char*>& arenas) {
@@ -718,7 +728,7 @@ int ep_dispatch_launch(ep_buffer_t* b, const ep_dispatch_args_t* pa) {
             return p;
         };
         EpLayoutArgs la{};
-        la.cnt_stride = (int)align_up(E / R + R, 4);
+        la.cnt_stride = (int)align_up(E / R + R, 8);
         la.col_total = carve(la.cnt_stride);
         la.blk_cnt = carve((int64_t)num_blocks * la.cnt_stride);
         if (R == 1) {
@@ -830,7 +840,7 @@ int ep_dispatch_recv_launch(ep_buffer_t* b, const ep_dispatch_recv_args_t* pa) {
             return p;
         };
         EpLayoutArgs la{};
-        la.cnt_stride = (int)align_up(E / R + R, 4);
+        la.cnt_stride = (int)align_up(E / R + R, 8);
         la.col_total = carve(la.cnt_stride);
         la.blk_cnt = carve((int64_t)num_blocks * la.cnt_stride);
         EP_HOST_ASSERT(off * (int64_t)sizeof(int) <= b->workspace_bytes and "layout scratch of the receive stream fits the workspace");
@@ -1271,7 +1281,7 @@ void ep_static_scratch_init() { (void)static_view_of_current_device(); }
 extern "C" int64_t ep_dispatch_static_scratch_bytes(int num_tokens, int num_topk, int num_experts) {
     if (num_tokens < 0 or num_topk <= 0 or num_experts <= 0) return -1;
     auto a64 = [](int64_t n) { return align_up(std::max<int64_t>(n, 1), 64); };
-    const int64_t W = align_up((int64_t)num_experts + 1, 4);
+    const int64_t W = align_up((int64_t)num_experts + 1, 8);
     const int64_t B = std::max<int64_t>(1, ceil_div(num_tokens, EP_TOKENS_PER_BLOCK));
     return EP_WS_HEADER_BYTES + 4 * (a64(W) + a64(B * W) + a64((int64_t)num_tokens * num_topk) + a64(num_tokens));
 }

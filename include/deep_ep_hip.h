@@ -243,7 +243,7 @@ int ep_dispatch_epilogue_launch(ep_buffer_t* buf, const ep_dispatch_epilogue_arg
  * array's address do allocate, and ep_init is where they happen.  The caller passes every input and output, the
  * outputs sized by ep_dispatch_worst_case_sizes(NULL, ...); epilogue_args->dispatch_stamp is ignored.  Fails
  * with a clear message when the scratch the shape needs, ep_dispatch_static_scratch_bytes(T, K, E) =
- * 4096 + 4 * (a64(W) + a64(B * W) + a64(T * K) + a64(T)) with W = E + 1 rounded up to 4, B = ceil(T / 128) (at
+ * 4096 + 4 * (a64(W) + a64(B * W) + a64(T * K) + a64(T)) with W = E + 1 rounded up to 8, B = ceil(T / 128) (at
  * least 1) and a64 rounding up to a multiple of 64, exceeds the array.  Results equal those of the two calls it
  * stands for.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (different streams,
  * or host threads) race; calls on one stream are ordered and safe. */

@@ -218,9 +218,11 @@ def test_deterministic_flag_gives_the_same_layout():
 
 
 @pytest.mark.parametrize('T,E,K,R,rank', [(700, 64, 6, 1, 0), (1500, 256, 8, 8, 3), (300, 2048, 4, 1, 0), (128, 256, 8, 1, 0),
-                                         (129, 256, 8, 4, 2)])
+                                         (129, 256, 8, 4, 2), (300, 2048, 8, 1, 0), (300, 2048, 32, 1, 0)])
 def test_single_and_multi_block_layouts_agree_with_oracle(T, E, K, R, rank):
-    """128 tokens fit one layout block (no counting pass runs); 129 need the counting and scan passes."""
+    """128 tokens fit one layout block (no counting pass runs); 129 need the counting pass.  2048 experts of one
+    partition are more count columns than the slot assignment that sums the counts itself has threads for: the scan
+    kernel runs at any size."""
     H, A = 128, 16
     topk, w = make_routing(T, E, K, seed=T, masked=0.1)
     lay = O.rank_share_layout(topk.numpy(), E, R, rank, A, T)
@@ -232,6 +234,25 @@ def test_single_and_multi_block_layouts_agree_with_oracle(T, E, K, R, rank):
                  'num_unaligned_recv_tokens_per_expert', 'dst_buffer_slot_idx', 'recv_src_metadata'):
         assert np.array_equal(getattr(handle, name).cpu().numpy(), lay[name]), name
     assert handle.num_recv_tokens_per_expert_list == lay['num_recv_tokens_per_expert_list']
+    buf.destroy()
+
+
+def test_block_counts_at_their_16_bit_bound():
+    """Every position of every token names expert 0: each of the 44 layout blocks counts 128 x 32 = 4096 entries for it,
+    the most a block can, and one thread of the slot assignment sums all 44 rows of that column (1024 experts: one row
+    stripe) in its 16-bit partial sums, 11 rows at a time."""
+    T, H, E, K, A = 5632, 128, 1024, 32, 16
+    topk = torch.zeros((T, K), dtype=torch.int64)
+    topk[::7, 3] = -1
+    w = torch.rand((T, K))
+    lay = O.rank_share_layout(topk.numpy(), E, 1, 0, A, T)
+    buf = _buffer(T, H, K)
+    _, _, _, handle, _ = buf.dispatch(make_tokens(T, H).to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV),
+                                      num_experts=E, expert_alignment=A, do_expand=True)
+    torch.cuda.synchronize()
+    for name in ('psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
+                 'num_unaligned_recv_tokens_per_expert', 'dst_buffer_slot_idx', 'recv_src_metadata'):
+        assert np.array_equal(getattr(handle, name).cpu().numpy(), lay[name]), name
     buf.destroy()
 
 
