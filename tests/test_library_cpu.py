@@ -48,6 +48,47 @@ def test_code_object_is_built_for_gfx950(de):
         assert k in blob, k
 
 
+def test_code_object_has_every_instance_of_the_slot_assignment(de):
+    blob = open(os.path.join(os.path.dirname(LIB), 'ep_kernels.hsaco'), 'rb').read()
+    for k in (b'ep_layout_assign_fold', b'ep_layout_assign_recv', b'ep_layout_assign_fold_recv'):
+        assert k in blob, k
+
+
+def test_slot_assignment_keeps_its_count_rows_in_flight(de, tmp_path):
+    """Two properties of the compiled kernels that the timings rest on and that a source change can lose without any
+    result changing, read from the compiler's assembly of the committed sources (same flags as the build):
+    no kernel reserves a private segment (no spills: the library's entry point for callers that cannot allocate must not
+    make the runtime set up scratch memory), and in the slot assignment that sums the block counts itself the 22 row
+    loads issued at the top are still in flight behind the staging of the ids and while the ids are counted per wave (the
+    compiler's wait-count pass merges the paths through the kernel: a wait for fewer outstanding loads there means that
+    the ids, or their counting, wait for the rows again)."""
+    import shutil
+    import subprocess
+    from deep_ep import _build
+    if shutil.which(_build.HIPCC) is None and not os.path.exists(_build.HIPCC):
+        pytest.skip('no hipcc here')
+    out = tmp_path / 'ep_kernels.s'
+    flags = [f for f in _build.DEVICE_FLAGS if f != '--genco']
+    subprocess.check_call([_build.HIPCC, *flags, '--cuda-device-only', '-S', '-o', str(out),
+                           os.path.join(_build.CSRC, 'ep_kernels.hip')], stderr=subprocess.DEVNULL)
+    text = out.read_text()
+    sizes = re.findall(r'\.amdhsa_private_segment_fixed_size (\d+)', text)
+    assert len(sizes) >= 30 and set(sizes) == {'0'}, sizes
+    body = text[text.index('\nep_layout_assign_fold:'):]
+    body = body[:body.index('.end_amdhsa_kernel')]
+    # in the order of the listing: ..., the ids waited for with the 22 row loads left outstanding, the barrier behind their
+    # staging, and the next wait for a load is the one for the first row, where the rows are summed
+    marks = []
+    for line in body.splitlines():
+        line = line.strip()
+        m = re.match(r's_waitcnt.*vmcnt\((\d+)\)', line)
+        if m:
+            marks.append(int(m.group(1)))
+        elif line.startswith('s_barrier'):
+            marks.append('barrier')
+    assert any(marks[i:i + 3] == [22, 'barrier', 21] for i in range(len(marks))), marks
+
+
 def test_size_calculators_match_oracle(de):
     C = de._C
     for (R, T, H, K, fp8) in [(1, 16384, 7168, 6, False), (1, 16384, 7168, 6, True), (32, 16384, 7168, 6, True),
