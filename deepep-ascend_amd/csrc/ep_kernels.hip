@@ -131,14 +131,14 @@ __device__ __forceinline__ int layout_num_rows(const EpLayoutArgs& a, int* s_psu
     return recv ? recv_scan_sources(a, s_psum) : a.num_tokens;
 }
 __device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s_key, short* s_rk, const int* s_psum,
-                                                 int num_rows, bool recv) {
+                                                 int num_rows, bool recv, int block) {
     const int K = a.num_topk;
     const int n = EP_TOKENS_PER_BLOCK * K;
     if (recv) {
         const int N = num_rows;
         for (int i = threadIdx.x; i < n; i += blockDim.x) {
             const int row = i / K, j = i - row * K;
-            const int g = blockIdx.x * EP_TOKENS_PER_BLOCK + row;
+            const int g = block * EP_TOKENS_PER_BLOCK + row;
             int e = -1;
             if (g < N) {
                 const int64_t pr = recv_packed_row(s_psum, a.num_ranks, a.max_tokens, g);
@@ -150,7 +150,7 @@ __device__ __forceinline__ void layout_load_keys(const EpLayoutArgs& a, short* s
         }
         return;
     }
-    const int64_t base = (int64_t)blockIdx.x * n;
+    const int64_t base = (int64_t)block * n;
     const int64_t total = (int64_t)a.num_tokens * K;
     if (total <= 0) {
         for (int i = threadIdx.x; i < n; i += blockDim.x) s_key[i] = s_rk[i] = -1;
@@ -200,7 +200,7 @@ extern "C" __global__ __launch_bounds__(EP_LAYOUT_THREADS) void ep_layout_count(
     const int num_rows = layout_num_rows(a, s_psum, a.recv_mode != 0);
     // the scan stops at the last workgroup that has rows: the ones behind it leave nothing
     if ((int)blockIdx.x > 0 && (int)blockIdx.x * EP_TOKENS_PER_BLOCK >= num_rows) return;
-    layout_load_keys(a, s_key, s_rk, s_psum, num_rows, a.recv_mode != 0);
+    layout_load_keys(a, s_key, s_rk, s_psum, num_rows, a.recv_mode != 0, blockIdx.x);
     __syncthreads();
     const int n = EP_TOKENS_PER_BLOCK * K;
     // (the position of an entry inside its token is carried along: a division by a run-time top-k is forty instructions)
@@ -319,11 +319,12 @@ __device__ __forceinline__ void layout_assign_body(const EpLayoutArgs& a) {
     const int lo = a.rank_idx * El;
     const int ncols = El + R;              // column c < El: local expert lo + c; else partition c - El
 
-    // With more than one block of tokens the launch has one workgroup more than blocks.  It ranks nothing: it sums the
-    // counts like the others and publishes the totals (handle tensors, inboxes, the host count page with its two
-    // system-scope fences), so that no ranking workgroup has that on its way.
+    // The launch has one workgroup more than blocks of tokens.  It ranks nothing: it gets the totals like the others
+    // (a single block: it counts that block's ids once more) and publishes them (handle tensors, inboxes, the host count
+    // page with its two system-scope fences), so that no ranking workgroup has that on its way.
     const bool single = !FOLD && a.scan_mode == EP_LAYOUT_SINGLE;     // (the summing instance never runs alone)
-    const bool publisher = single || b == a.num_blocks, worker = single || b < a.num_blocks;
+    const bool publisher = b == a.num_blocks, worker = !publisher;
+    const int kb = single ? 0 : b;         // the block whose ids this workgroup stages
     const int num_rows = layout_num_rows(a, s_psum, RECV);
     if (!publisher && b > 0 && b * EP_TOKENS_PER_BLOCK >= num_rows) return;      // nothing to rank here
 
@@ -342,7 +343,7 @@ __device__ __forceinline__ void layout_assign_body(const EpLayoutArgs& a) {
     }
     // This workgroup's expert ids are asked for first (send side, up to four ids a thread).
     const int nkeys = EP_TOKENS_PER_BLOCK * K;
-    const int64_t key_base = (int64_t)b * nkeys, key_total = (int64_t)a.num_tokens * K;
+    const int64_t key_base = (int64_t)kb * nkeys, key_total = (int64_t)a.num_tokens * K;
     const bool folded = FOLD;
     const bool keys_early = folded && !RECV && nkeys <= 4 * EP_LAYOUT_THREADS && key_total > 0;
     // EP_LAYOUT_FOLDED: ep_layout_count has finished and left plain counts as 16-bit halves; the rows before this
@@ -436,7 +437,7 @@ __device__ __forceinline__ void layout_assign_body(const EpLayoutArgs& a) {
         }
     } else {
         clear_counters();
-        layout_load_keys(a, s_key, s_rk, s_psum, num_rows, RECV);
+        layout_load_keys(a, s_key, s_rk, s_psum, num_rows, RECV, kb);
         if (FOLD) fold_loads(v_first, s0, min(g0, FG - 1));
     }
     __syncthreads();

@@ -298,9 +298,9 @@ void launch_layout(EpLayoutArgs& la, int num_blocks, void* stream) {
         launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, layout_count_lds(E, R, K), stream, la);
     if (la.scan_mode == EP_LAYOUT_SCANNED)
         launch(g_k.layout_scan, (unsigned)ceil_div(la.cnt_stride, 16), EP_SCAN_THREADS, 0, stream, la);
-    // (several blocks: one workgroup more, which publishes the totals and ranks nothing)
-    launch(g_k.layout_assign[la.scan_mode == EP_LAYOUT_FOLDED][la.recv_mode != 0],
-           (unsigned)num_blocks + (la.scan_mode == EP_LAYOUT_SINGLE ? 0u : 1u), EP_LAYOUT_THREADS, smem_assign, stream, la);
+    // (one workgroup more than blocks: it publishes the totals and ranks nothing)
+    launch(g_k.layout_assign[la.scan_mode == EP_LAYOUT_FOLDED][la.recv_mode != 0], (unsigned)num_blocks + 1u, EP_LAYOUT_THREADS,
+           smem_assign, stream, la);
 }
 
 void write_peer_table(ep_buffer* b, const std::vector<char*>& arenas) {
