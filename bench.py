@@ -198,6 +198,36 @@ def dispatch_ceiling(ep_calib, timed, n, cargs, us_scatter):
             'kernels': 'ep_calib_scatter_stores_only, ep_calib_read_rows (ep_calib.hsaco), isolated flushed medians'}
 
 
+def calib_combine_args(ep_calib, y, recv_w, handle, combined_x, combined_w, T, H, K, E, blocks_per_cu):
+    """The combine of this run as the calibration library's kernels take it."""
+    a = ep_calib.CombineArgs()
+    num_recv = handle.psum_num_recv_tokens_per_rank[-1:]
+    keep = (y, recv_w, handle.recv_src_metadata, num_recv, handle.topk_idx, combined_x, combined_w)
+    a.y, a.expanded_weights = y.data_ptr(), recv_w.data_ptr()
+    a.recv_src_metadata, a.num_recv, a.topk_idx = handle.recv_src_metadata.data_ptr(), num_recv.data_ptr(), handle.topk_idx.data_ptr()
+    a.combined_x, a.combined_topk_weights = combined_x.data_ptr(), combined_w.data_ptr()
+    a.num_tokens, a.hidden, a.num_topk, a.num_experts = T, H, K, E
+    a.num_recv_rows, a.num_in_rows, a.blocks_per_cu = handle.recv_src_metadata.size(0), y.size(0), blocks_per_cu
+    return a, keep
+
+
+def combine_ceiling(ep_calib, timed, n, cargs, us_combine):
+    """The combine kernel taken apart the same way: its row fetches (with the sums) alone and its stores alone, from
+    two kernels of the calibration code object that run the product's kernel body.  The fetches run as the product is
+    launched (workgroups a CU capped); the stores alone are timed uncapped: capped, that launch waits on its slot
+    lookups (about 100 us) and says nothing about the store stream."""
+    med = lambda v: v[len(v) // 2]  # noqa: E731
+    ld = med(timed(lambda: ep_calib.combine('combine_loads_only', cargs), n))
+    cap = cargs.blocks_per_cu
+    cargs.blocks_per_cu = 0
+    st = med(timed(lambda: ep_calib.combine('combine_stores_only', cargs), n))
+    cargs.blocks_per_cu = cap
+    return {'loads_only_us': round(ld, 2), 'stores_only_us': round(st, 2), 'sum_us': round(ld + st, 2),
+            'combine_kernel_us': round(us_combine, 2), 'combine_kernel_over_sum': round(us_combine / (ld + st), 3),
+            'kernels': f'ep_calib_combine_k6_loads_only ({cap} workgroups a CU, as the library launches its own), '
+                       'ep_calib_combine_k6_stores_only (uncapped) (ep_calib.hsaco), isolated flushed medians'}
+
+
 def calibrate_write(ep_calib, timed, n, cargs, T, H, K, n_valid, n_recv, pad_bytes, dev, us_scatter, meta):
     """Pure writes of the byte count the fused FP8 copy kernel writes (payload, scales, weights, zero padding),
     same sampling as the kernels: 4 KiB chunks in address order, in scrambled order, 256 write fronts in lock
@@ -754,6 +784,14 @@ def main():
         ep_calib.init()
         cargs, keep = calib_scatter_args(ep_calib, xg, wg, handle, recv[0], recv[1], recv_w, T, H, K, E, A)
         roofline['dispatch_ceiling'] = dispatch_ceiling(ep_calib, timed, n_k, cargs, us_scatter)
+        if K == 6:
+            # the same for the combine kernel (isolated flushed median against its two streams alone)
+            blocks_per_cu = 3 if args.combine_blocks_per_cu is None or args.combine_blocks_per_cu < 0 else args.combine_blocks_per_cu
+            cx = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+            cw = torch.empty((T, K), dtype=torch.float32, device=dev)
+            ccargs, ckeep = calib_combine_args(ep_calib, y, recv_w, handle, cx, cw, T, H, K, E, blocks_per_cu)
+            roofline['combine_ceiling'] = combine_ceiling(ep_calib, timed, n_k, ccargs, med(t_combine))
+            del ckeep, cx, cw
         if args.calibrate_write:
             out['write_calibration'] = calibrate_write(ep_calib, timed, n_k, cargs, T, H, K, n_valid, n_recv, pad_bytes,
                                                        dev, us_scatter, handle.recv_src_metadata)

@@ -66,10 +66,15 @@ const char* const kVariantKernels[kNumVariants] = {
     "ep_calib_ordered_steered", "ep_calib_ordered_steered_stores_only", "ep_calib_ordered_steered_loads_only",
     "ep_calib_quant_rows", "ep_calib_copy_ordered_flat", "ep_calib_copy_ordered_steered"};
 
+constexpr int kNumCombineVariants = 3;
+const char* const kCombineKernels[kNumCombineVariants] = {"ep_calib_combine_k6", "ep_calib_combine_k6_loads_only",
+                                                          "ep_calib_combine_k6_stores_only"};
+
 struct Kernels {
     hipModule_t module = nullptr;
     hipFunction_t fill, fill_shuffled, fill_affine, fronts, mixed;
     hipFunction_t variant[kNumVariants];
+    hipFunction_t combine[kNumCombineVariants];
     int device = -1;
 };
 std::mutex g_mutex;
@@ -100,13 +105,14 @@ void load_kernels(const char* dir) {
     get(g_k.fronts, "ep_calib_fronts");
     get(g_k.mixed, "ep_calib_mixed");
     for (int i = 0; i < kNumVariants; ++i) get(g_k.variant[i], kVariantKernels[i]);
+    for (int i = 0; i < kNumCombineVariants; ++i) get(g_k.combine[i], kCombineKernels[i]);
     g_k.module = m;
 }
 
 template <class A>
-void launch(hipFunction_t fn, unsigned grid, unsigned block, void* stream, A& args) {
+void launch(hipFunction_t fn, unsigned grid, unsigned block, void* stream, A& args, unsigned lds_bytes = 0) {
     void* params[] = {&args};
-    HIP_CHECK(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, 0, (hipStream_t)stream, params, nullptr));
+    HIP_CHECK(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, lds_bytes, (hipStream_t)stream, params, nullptr));
 }
 
 void check_device() {
@@ -274,6 +280,52 @@ int ep_calib_scatter(int variant, const ep_calib_scatter_t* pa) {
         oa.s = sa;
         const bool writes = variant != EP_CALIB_ORDERED_STEERED_LOADS_ONLY;
         launch(g_k.variant[variant], (unsigned)row_blocks + (writes ? pad_blocks : 0u), EP_ROW_THREADS, c.stream, oa);
+    });
+}
+
+int ep_calib_combine(int variant, const ep_calib_combine_t* pa) {
+    return guarded([&] {
+        load_kernels(nullptr);
+        check_device();
+        CALIB_ASSERT(pa != nullptr);
+        CALIB_ASSERT(variant >= 0 and variant < kNumCombineVariants);
+        const ep_calib_combine_t& c = *pa;
+        const int T = c.num_tokens, H = c.hidden, K = c.num_topk;
+        CALIB_ASSERT(K == 6 and T > 0 and H > 0 and H % 8 == 0 and c.num_experts > 0 and c.num_experts <= EP_MAX_EXPERTS);
+        CALIB_ASSERT(c.num_recv_rows > 0 and c.num_recv_rows <= T and c.num_in_rows > 0);
+        CALIB_ASSERT(c.y != nullptr and c.recv_src_metadata != nullptr and c.num_recv != nullptr and c.topk_idx != nullptr);
+        CALIB_ASSERT(c.combined_x != nullptr and ((uintptr_t)c.y & 15) == 0 and ((uintptr_t)c.combined_x & 15) == 0);
+        CALIB_ASSERT((c.expanded_weights == nullptr) == (c.combined_topk_weights == nullptr));
+        CALIB_ASSERT(c.blocks_per_cu >= 0);
+
+        EpCombineArgs ca{};
+        ca.y = c.y;
+        ca.expanded_weights = c.expanded_weights;
+        ca.recv_src_metadata = c.recv_src_metadata;
+        ca.num_recv_ptr = c.num_recv;
+        ca.topk_idx = c.topk_idx;
+        ca.combined_x = c.combined_x;
+        ca.combined_topk_weights = c.combined_topk_weights;
+        ca.hidden = H;
+        ca.num_topk = K;
+        ca.num_tokens = T;
+        ca.num_rows_bound = c.num_recv_rows;
+        ca.rank_idx = 0;
+        ca.max_tokens = T;
+        ca.num_experts = c.num_experts;
+        ca.num_parts = (int)std::max<int64_t>(1, ceil_div(H, 1024));
+        ca.y_row_bytes = (int64_t)H * 2;
+        ca.out_row_bytes = (int64_t)H * 2;
+        ca.num_ranks = 1;
+        ca.experts_per_rank = c.num_experts;
+        ca.num_in_rows = c.num_in_rows;
+        ca.num_groups = 1;
+        ca.num_row_blocks = (int)ceil_div((int64_t)ca.num_rows_bound * ca.num_parts, EP_ROWS_PER_BLOCK);
+        const unsigned grid = (unsigned)ca.num_row_blocks + (unsigned)ceil_div(T, EP_ROW_THREADS);
+        // an unused LDS allocation caps the workgroups a compute unit holds (160 KiB of LDS a CU), as the library does
+        unsigned lds = 0;
+        if (c.blocks_per_cu >= 2 and c.blocks_per_cu < 160) lds = std::min(64u * 1024u, 160u * 1024u / (unsigned)c.blocks_per_cu - 1024u);
+        launch(g_k.combine[variant], grid, EP_ROW_THREADS, c.stream, ca, lds);
     });
 }
 

@@ -13,6 +13,7 @@
 //                                      all readers of a token on one XCD, so that x is fetched from memory once
 //   ep_calib_quant_rows + ep_calib_copy_ordered_{flat,steered}   the same in two passes: quantise token-major,
 //                                      then copy FP8 rows in destination order
+//   ep_calib_combine_k6*               the single-partition combine at top-6: whole, its row fetches alone, its stores alone
 #include "ep_kernels.hip"
 #include "ep_calib_args.h"
 
@@ -241,3 +242,15 @@ __device__ __forceinline__ void copy_ordered_body(const EpCalibOrderedArgs& o) {
 }
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_calib_copy_ordered_flat(EpCalibOrderedArgs o) { copy_ordered_body<false>(o); }
 extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_calib_copy_ordered_steered(EpCalibOrderedArgs o) { copy_ordered_body<true>(o); }
+
+// The single-partition combine at top-6 whole, without its stores, and without its row fetches: what the gather
+// and the store stream of the product kernel cost alone.
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_calib_combine_k6(EpCombineArgs a) {
+    combine_body<6, EP_COMBINE_FUSED>(a);
+}
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_calib_combine_k6_loads_only(EpCombineArgs a) {
+    combine_body<6, EP_COMBINE_FUSED, true, false>(a);
+}
+extern "C" __global__ __launch_bounds__(EP_ROW_THREADS) void ep_calib_combine_k6_stores_only(EpCombineArgs a) {
+    combine_body<6, EP_COMBINE_FUSED, false, true>(a);
+}

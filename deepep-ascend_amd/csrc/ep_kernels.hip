@@ -1212,8 +1212,11 @@ __device__ __forceinline__ void combine_unrouted(const EpCombineArgs& a) {
 //                       (last top-k position per destination partition) in ascending position, summed
 //                       left to right in fp32 and rounded once; weight vectors OR-merged
 //                       (combine_reduce_epilogue.hpp:96-153)
-template <int KT, int MODE>
+// LOADS / STORES: the benchmarks' calibration code object builds the single-partition kernel once without its row
+// fetches and once without its stores (what each stream costs alone); the library's kernels have both.
+template <int KT, int MODE, bool LOADS = true, bool STORES = true>
 __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
+    static_assert((LOADS && STORES) || (KT > 0 && MODE == EP_COMBINE_FUSED), "only the unrolled single-partition kernel is taken apart");
     if (MODE == EP_COMBINE_FUSED && (int)blockIdx.x >= a.num_row_blocks) {
         combine_unrouted(a);
         return;
@@ -1296,9 +1299,9 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
         }
     } else {
         const bool need_w = part == 0 || (MODE == EP_COMBINE_FUSED && a.weighted);
-        if (need_w && a.expanded_weights != nullptr && myslot >= 0) myw = a.expanded_weights[myslot];
+        if (LOADS && need_w && a.expanded_weights != nullptr && myslot >= 0) myw = a.expanded_weights[myslot];
         if (part == 0 && lane < K) {
-            if (MODE == EP_COMBINE_FUSED && a.combined_topk_weights != nullptr)
+            if (STORES && MODE == EP_COMBINE_FUSED && a.combined_topk_weights != nullptr)
                 a.combined_topk_weights[(int64_t)t * K + lane] = myw;
             // (the verbatim path below stores them behind its row fetches, so that the two trips become one)
             if (MODE == EP_COMBINE_PARTIAL && a.expanded_weights != nullptr && !verbatim)
@@ -1370,6 +1373,10 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
                 d0[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + c0);
                 d1[j] = __builtin_nontemporal_load(y + (int64_t)s * yvec + c1);
             }
+        } else if (!LOADS) {
+            const u32x4 filler = {(unsigned)lane, (unsigned)i, 0x3f803f80u, 0x3f803f80u};
+#pragma unroll
+            for (int j = 0; j < KT; ++j) d0[j] = d1[j] = filler;
         } else if (nvalid > 0) {
             // nearly every position is valid: one straight run of 2 K loads with no branch in it, a position without
             // a row re-reads the first valid one (the same cache lines again) and is left out of the sum below
@@ -1419,15 +1426,16 @@ __device__ __forceinline__ void combine_body(const EpCombineArgs& a) {
             if (nin >= 2 || (weighted && nin == 1)) return pack8(acc);
             return first;
         };
+        // (without stores the sums still have to be formed: they are stored under a condition that never holds)
         if (live0) {
             u32x4 res = reduce(p0a, p1a, d0);
             if (MODE == EP_COMBINE_FUSED) res = add_loaded_biases(has0, p0a, has1, p1a, res);
-            stream_store<EP_COMBINE_ST_POL>(out + v0, res);
+            if (STORES || ((res.x ^ res.y ^ res.z ^ res.w) == 0x9E3779B1u && a.num_in_rows < 0)) stream_store<EP_COMBINE_ST_POL>(out + v0, res);
         }
         if (live1) {
             u32x4 res = reduce(p0b, p1b, d1);
             if (MODE == EP_COMBINE_FUSED) res = add_loaded_biases(has0, p0b, has1, p1b, res);
-            stream_store<EP_COMBINE_ST_POL>(out + v1, res);
+            if (STORES || ((res.x ^ res.y ^ res.z ^ res.w) == 0x9E3779B1u && a.num_in_rows < 0)) stream_store<EP_COMBINE_ST_POL>(out + v1, res);
         }
         continue;
     }

@@ -26,6 +26,17 @@ class ScatterArgs(ctypes.Structure):
             'do_zero_padding', 'num_entries', 'entries_per_list', 'num_lists')] + [('stream', ctypes.c_void_p)]
 
 
+COMBINE_VARIANTS = ('combine', 'combine_loads_only', 'combine_stores_only')
+
+
+class CombineArgs(ctypes.Structure):
+    # ep_calib_combine_t
+    _fields_ = [(n, ctypes.c_void_p) for n in (
+        'y', 'expanded_weights', 'recv_src_metadata', 'num_recv', 'topk_idx', 'combined_x', 'combined_topk_weights')] + [
+            (n, ctypes.c_int32) for n in ('num_tokens', 'hidden', 'num_topk', 'num_experts', 'num_recv_rows', 'num_in_rows',
+                                          'blocks_per_cu', 'reserved')] + [('stream', ctypes.c_void_p)]
+
+
 def _sig(name, *argtypes):
     fn = getattr(_lib, name)
     fn.restype = ctypes.c_int
@@ -43,6 +54,7 @@ _fronts = _sig('ep_calib_fronts', ctypes.c_void_p, ctypes.c_int, ctypes.c_int, c
 _mixed = _sig('ep_calib_mixed', ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_uint,
               ctypes.c_void_p)
 _scatter = _sig('ep_calib_scatter', ctypes.c_int, ctypes.POINTER(ScatterArgs))
+_combine = _sig('ep_calib_combine', ctypes.c_int, ctypes.POINTER(CombineArgs))
 
 
 class CalibError(RuntimeError):
@@ -91,6 +103,13 @@ def mixed(src: torch.Tensor, dst: torch.Tensor, reads_num: int, reads_den: int) 
 def scatter(variant: str, args: ScatterArgs) -> None:
     args.stream = _stream()
     _check(_scatter(VARIANTS.index(variant), ctypes.byref(args)))
+
+
+def combine(variant: str, args: CombineArgs) -> None:
+    """The single-partition combine at top-6: 'combine' (the product's kernel body), 'combine_loads_only' (its row
+    fetches and sums, nothing written), 'combine_stores_only' (its stores of filler rows, nothing fetched but the slots)."""
+    args.stream = _stream()
+    _check(_combine(COMBINE_VARIANTS.index(variant), ctypes.byref(args)))
 
 
 def build_order(recv_src_metadata: torch.Tensor, num_topk: int, chunk_tokens: int, steered: bool):

@@ -1,8 +1,8 @@
 /* C ABI of libdeep_ep_calib.so -- the measurement rig of the benchmarks for the MI355X EP dispatch path.
  * It is NOT part of the product: libdeep_ep_hip.so neither links nor loads it, and nothing in it has a
  * counterpart in the reference.  It owns a code object of its own (ep_calib.hsaco, next to the library)
- * with pure-write patterns, the product's fused copy kernel with its loads or its stores taken out, and
- * the destination-ordered and two-pass formulations of that kernel, so that every figure a benchmark
+ * with pure-write patterns, the product's fused copy kernel and its combine kernel with their loads or their
+ * stores taken out, and the destination-ordered and two-pass formulations of the copy kernel, so that every figure a benchmark
  * quotes for "what the memory system allows" comes from a committed kernel run in the same process.
  * Every function returns 0 on success; otherwise ep_calib_last_error() holds a thread-local message.
  * Nothing here allocates or synchronises; all kernels are enqueued on `stream`. */
@@ -82,6 +82,31 @@ typedef struct ep_calib_scatter {
 /* Enqueues one variant.  H must be a multiple of 128 (a multiple of 512 and at most 7168 for the two-pass
  * variants), T at most 2^24 - 1, K at most 32. */
 int ep_calib_scatter(int variant, const ep_calib_scatter_t* args);
+
+enum ep_calib_combine_variant {
+    EP_CALIB_COMBINE = 0,               /* the product's single-partition combine body at top-6 */
+    EP_CALIB_COMBINE_LOADS_ONLY = 1,    /* ... its row fetches and sums alone (nothing is written) */
+    EP_CALIB_COMBINE_STORES_ONLY = 2    /* ... its stores alone (rows of filler values; nothing is fetched but the slots) */
+};
+
+typedef struct ep_calib_combine {
+    /* a single-partition BF16 combine at top-6 without biases, as the product's kernel takes it */
+    const void* y;                      /* [num_in_rows, H] BF16 expert outputs */
+    const float* expanded_weights;      /* [num_in_rows] or NULL */
+    const int32_t* recv_src_metadata;   /* [num_recv_rows, K + 2] of the dispatch handle */
+    const int32_t* num_recv;            /* device scalar: received rows */
+    const int64_t* topk_idx;            /* [T, K] */
+    void* combined_x;                   /* [T, H] BF16 out */
+    float* combined_topk_weights;       /* [T, K] out, or NULL (iff expanded_weights is NULL) */
+    int32_t num_tokens, hidden, num_topk, num_experts;
+    int32_t num_recv_rows, num_in_rows;
+    int32_t blocks_per_cu;              /* workgroups a compute unit holds at once (0: no cap); the library's own choice at top-6 is 3 */
+    int32_t reserved;
+    void* stream;
+} ep_calib_combine_t;
+
+/* Enqueues one variant.  K must be 6, H a multiple of 8. */
+int ep_calib_combine(int variant, const ep_calib_combine_t* args);
 
 #ifdef __cplusplus
 }

@@ -80,6 +80,58 @@ def test_calibration_variants_reproduce_the_product_output(T, H, E, K, A, masked
     buf.destroy()
 
 
+@pytest.mark.parametrize('T,H,E,A,masked', [(1024, 2048, 32, 16, 0.0), (700, 7168, 64, 128, 0.2)])
+def test_calibration_combine_reproduces_the_product_output(T, H, E, A, masked):
+    """The combine kernel body as the calibration code object builds it (top-6) gives the product's bytes; its
+    loads-only form writes nothing; its stores-only form writes every row the product writes."""
+    import deep_ep
+    import ep_calib
+    ep_calib.init()
+    K = 6
+    dev = torch.device('cuda', 0)
+    x = make_tokens(T, H, seed=9).to(dev)
+    topk, w = make_routing(T, E, K, seed=9, masked=masked)
+    topk, w = topk.to(dev), w.to(dev)
+    buf = deep_ep.EPBuffer(deep_ep.LocalGroup(), num_max_tokens_per_rank=T, hidden=H, num_topk=K, explicitly_destroy=True)
+    rx, _, rw, handle, _ = buf.dispatch(x, topk_idx=topk, topk_weights=w, num_experts=E, expert_alignment=A,
+                                        do_expand=True, do_zero_padding=True)
+    y = (rx.float() * 0.5 + 0.25).to(torch.bfloat16)
+    want_x, want_w, _ = buf.combine(y, handle, topk_weights=rw)
+    torch.cuda.synchronize()
+    num_recv = handle.psum_num_recv_tokens_per_rank[-1:]
+
+    def args_for(ox, ow):
+        a = ep_calib.CombineArgs()
+        a.y, a.expanded_weights = y.data_ptr(), rw.data_ptr()
+        a.recv_src_metadata, a.num_recv, a.topk_idx = handle.recv_src_metadata.data_ptr(), num_recv.data_ptr(), topk.data_ptr()
+        a.combined_x, a.combined_topk_weights = ox.data_ptr(), ow.data_ptr()
+        a.num_tokens, a.hidden, a.num_topk, a.num_experts = T, H, K, E
+        a.num_recv_rows, a.num_in_rows, a.blocks_per_cu = handle.recv_src_metadata.size(0), y.size(0), 3
+        return a
+
+    ox, ow = torch.full_like(want_x, 7.0), torch.full_like(want_w, 7.0)
+    ep_calib.combine('combine', args_for(ox, ow))
+    torch.cuda.synchronize()
+    assert torch.equal(ox.view(torch.int16), want_x.view(torch.int16)) and torch.equal(ow.view(torch.int32), want_w.view(torch.int32))
+    # loads only: the rows of routed tokens stay as they were (tokens without any expert are zeroed by the workgroups
+    # that look after them in every form)
+    routed = (topk >= 0).any(dim=1)
+    ox.fill_(7.0)
+    ep_calib.combine('combine_loads_only', args_for(ox, ow))
+    torch.cuda.synchronize()
+    assert bool((ox[routed] == 7.0).all())
+    # stores only: every routed token's row is written
+    ox.fill_(7.0)
+    ep_calib.combine('combine_stores_only', args_for(ox, ow))
+    torch.cuda.synchronize()
+    assert not bool((ox[routed] == 7.0).all(dim=1).any())
+    with pytest.raises(ep_calib.CalibError, match='Assertion exception'):
+        a = args_for(ox, ow)
+        a.num_topk = 4
+        ep_calib.combine('combine', a)
+    buf.destroy()
+
+
 def test_calibration_fills_write_every_byte():
     import ep_calib
     ep_calib.init()
