@@ -113,6 +113,7 @@ struct DispatchState {
     int num_tokens, hidden, num_topk, num_local_experts;
     int num_max_tokens_per_rank, num_experts, expert_alignment;
     bool cached_mode, do_cpu_sync, do_zero_padding, use_col_major_sf, fused;
+    bool exact_sync_sizes = false;
 };
 
 py::tuple run_dispatch_epilogue(DispatchState& s) {
@@ -163,13 +164,15 @@ py::tuple run_dispatch_epilogue(DispatchState& s) {
         num_expanded = (int)s.cached_num_expanded;
         alloc_recv = num_recv;
         alloc_expanded = num_expanded;
-    } else if (s.do_cpu_sync && s.connected) {
+    } else if (s.do_cpu_sync && (s.connected || s.exact_sync_sizes)) {
         // a node: the bound over every partition's tokens is far above what arrives; wait for the counts
+        // (one partition, on request: outputs of exactly the counted sizes, as the reference allocates them, at the
+        // price of an idle GPU between the layout kernels and the copy)
         wait_counts();
         counts_from_host = true;
         alloc_recv = num_recv;
         alloc_expanded = num_expanded;
-        meta = meta.narrow(0, 0, num_recv);
+        if (have_meta) meta = meta.narrow(0, 0, num_recv);
     } else if (s.do_cpu_sync) {
         // Exact sizes come from the host count page, but waiting for it here would leave the GPU idle between the
         // layout kernels and the copy.  Allocate for this call's upper bound, enqueue the copy, and read the counts
@@ -290,6 +293,7 @@ public:
         : buf_((ep_buffer_t*)handle), rank_idx_(rank_idx), num_ranks_(num_ranks) {}
 
     void set_connected(bool c) { connected_ = c; }
+    void set_exact_sync_sizes(bool e) { exact_sync_sizes_ = e; }
     void invalidate() { buf_ = nullptr; }
 
     // argument order of csrc/buffers/ep.hpp:89-112
@@ -323,6 +327,7 @@ public:
         s.buf = buf_;
         s.num_ranks = num_ranks_;
         s.connected = connected_;
+        s.exact_sync_sizes = exact_sync_sizes_;
         s.x = x;
         s.sf = sf;
         s.topk_idx = topk_idx;
@@ -452,6 +457,7 @@ private:
     ep_buffer_t* buf_;
     int rank_idx_, num_ranks_;
     bool connected_ = false;
+    bool exact_sync_sizes_ = false;
 };
 
 }  // namespace
@@ -462,6 +468,7 @@ PYBIND11_MODULE(_native, m) {
     py::class_<NativeBuffer>(m, "Buffer")
         .def(py::init<uintptr_t, int, int>())
         .def("set_connected", &NativeBuffer::set_connected)
+        .def("set_exact_sync_sizes", &NativeBuffer::set_exact_sync_sizes)
         .def("invalidate", &NativeBuffer::invalidate)
         .def("dispatch", &NativeBuffer::dispatch, py::arg("x"), py::arg("sf"), py::arg("topk_idx"), py::arg("topk_weights"),
              py::arg("cumulative_local_expert_recv_stats"), py::arg("cached_num_recv_tokens"),

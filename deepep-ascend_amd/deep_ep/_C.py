@@ -349,6 +349,12 @@ class EPBuffer(BufferBase):
         else:
             self.lb_storage = torch.empty(0, dtype=torch.uint8, device=self.device)
 
+    def set_exact_sync_sizes(self, enable: bool) -> None:
+        """Host-synchronised dispatches of a single partition wait for the counts before they allocate (outputs of
+        exactly the counted sizes, as csrc/buffers/ep.hpp:300-351 allocates them) instead of allocating for the call's
+        upper bound and narrowing."""
+        self._native.set_exact_sync_sizes(bool(enable))
+
     # ---- lifecycle ----
     def destroy(self) -> None:
         if self.destroyed:

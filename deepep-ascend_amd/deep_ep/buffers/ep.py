@@ -156,6 +156,14 @@ class EPBuffer(BufferBase):
         super().destroy()
         self.context = self.hccl_comm_handle = None
 
+    def set_exact_sync_sizes(self, enable: bool = True) -> None:
+        """No counterpart in the reference (an allocation policy of this library).  By default a dispatch with
+        `do_cpu_sync=True` on a single partition allocates its outputs for the call's upper bound, enqueues the copy at
+        once and returns views narrowed to the exact sizes, which keep the bound-sized storage alive.  With this switch
+        on, such a dispatch waits for the counts first and allocates exactly what its results show, as the reference
+        does; the GPU then idles between the layout kernels and the copy (about 10 microseconds a call)."""
+        self.runtime.set_exact_sync_sizes(enable)
+
     @staticmethod
     def get_buffer_size_hint(group, num_max_tokens_per_rank: int, hidden: int, num_topk: int = 0,
                              use_fp8_dispatch: bool = False, allow_hybrid_mode: bool = True,
@@ -213,7 +221,7 @@ class EPBuffer(BufferBase):
                 before the host has the counts, and are returned as views narrowed to the exact
                 sizes: while such a view is alive it keeps the whole bound-sized allocation (up to
                 about 15 % more rows than its shape shows under uniform routing); `.clone()` it to
-                hold only the rows shown.  An epilogue deferred with `defer_epilogue` must run
+                hold only the rows shown, or call `set_exact_sync_sizes()` on the buffer once.  An epilogue deferred with `defer_epilogue` must run
                 before the next non-cached dispatch is launched on this buffer: the library
                 refuses an epilogue whose dispatch is no longer the buffer's latest.
             do_expand: must be True.  do_handle_copy must be False.

@@ -279,6 +279,34 @@ def test_folded_and_scanned_block_prefixes_agree(T, E, K, R, rank):
         deep_ep._C.set_layout_fold_max_blocks(256)
 
 
+@pytest.mark.parametrize('fused', [False, True])
+def test_exact_sync_sizes_allocate_what_the_results_show(fused):
+    """A host-synchronised dispatch returns views of bound-sized storage by default; with `set_exact_sync_sizes()` the
+    storage is exactly what the shapes show, and the results are the same bytes."""
+    T, H, E, K, A = 777, 512, 32, 4, 64
+    topk, w = make_routing(T, E, K, seed=3, masked=0.2)
+    x = make_tokens(T, H, seed=3)
+    buf = _buffer(T, H, K, use_fp8_dispatch=fused)
+    kw = dict(topk_idx=topk.to(DEV), topk_weights=w.to(DEV), num_experts=E, expert_alignment=A, do_expand=True,
+              do_zero_padding=True, fused_fp8_quant=fused)
+    r0, _, w0, h0, _ = buf.dispatch(x.to(DEV), **kw)
+    buf.set_exact_sync_sizes(True)
+    r1, _, w1, h1, _ = buf.dispatch(x.to(DEV), **kw)
+    buf.set_exact_sync_sizes(False)
+    torch.cuda.synchronize()
+    p0, p1 = (r0[0], r1[0]) if fused else (r0, r1)
+    assert p1.shape == p0.shape and p1.untyped_storage().nbytes() == p1.numel() * p1.element_size()
+    assert p0.untyped_storage().nbytes() > p0.numel() * p0.element_size()
+    assert w1.untyped_storage().nbytes() == w1.numel() * 4
+    assert h1.recv_src_metadata.untyped_storage().nbytes() == h1.recv_src_metadata.numel() * 4
+    assert torch.equal(p0.view(torch.uint8), p1.view(torch.uint8)) and torch.equal(w0, w1)
+    if fused:
+        assert torch.equal(r0[1], r1[1]) and r1[1].untyped_storage().nbytes() == r1[1].numel() * 4
+    assert torch.equal(h0.recv_src_metadata, h1.recv_src_metadata)
+    assert h0.num_recv_tokens_per_expert_list == h1.num_recv_tokens_per_expert_list
+    buf.destroy()
+
+
 def test_epilogue_of_an_overtaken_dispatch_is_refused():
     """Two deferred dispatches on one buffer: the second launch overwrites the slot map in the buffer's
     workspace, so the first one's copy epilogue must not run any more; the host refuses it."""
