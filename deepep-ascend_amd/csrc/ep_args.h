@@ -17,6 +17,8 @@
 #define EP_LAYOUT_SCANNED 0
 #define EP_LAYOUT_FOLDED 1
 #define EP_LAYOUT_SINGLE 2
+#define EP_LAYOUT_RECOUNTED 3     // no kernel in front: every workgroup counts the ids of all (few) blocks itself
+#define EP_RECOUNT_DEPTH 24       // ids a thread of the slot assignment holds in flight for that (blocks x top-k <= 2 x this)
 
 #define EP_SCATTER_EXPAND 0
 #define EP_SCATTER_PACK 1

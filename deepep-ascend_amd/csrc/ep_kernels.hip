@@ -294,6 +294,8 @@ extern "C" __global__ __launch_bounds__(EP_SCAN_THREADS) void ep_layout_scan(EpL
 //   EP_LAYOUT_FOLDED   ep_layout_count left plain counts in blk_cnt (16-bit halves): every block sums the rows
 //                      before it itself (cheaper than a launch of its own up to a few hundred blocks)
 //   EP_LAYOUT_SINGLE   one block owns every token: nothing ran before, its own LDS counts are the totals
+//   EP_LAYOUT_RECOUNTED  a few blocks of one partition: nothing ran before, every workgroup counts the ids of all
+//                      blocks itself (a launch less; the ids of 1024 tokens are 48 KB)
 // Only the local experts and the partitions need prefixes: slots of other experts are never used.
 // ------------------------------------------------------------------------------------------------
 #define EP_FOLD_DEPTH 22
@@ -341,9 +343,83 @@ __device__ __forceinline__ void layout_assign_body(const EpLayoutArgs& a) {
             tot[k] = a.col_total[c];
         }
     }
-    // This workgroup's expert ids are asked for first (send side, up to four ids a thread).
     const int nkeys = EP_TOKENS_PER_BLOCK * K;
     const int64_t key_base = (int64_t)kb * nkeys, key_total = (int64_t)a.num_tokens * K;
+    // EP_LAYOUT_RECOUNTED (one partition, a few blocks, send side): every workgroup reads the ids of all blocks in one
+    // go: a histogram of all of them (the totals), one of the blocks before its own, its own block's ids staged on the
+    // way.  With one partition the master of a token is its last valid position: the partition's column counts the
+    // tokens that have a valid id at all (flags in LDS, counted by ballot).
+    const bool recount = !FOLD && !RECV && a.scan_mode == EP_LAYOUT_RECOUNTED;
+    if (recount) {
+        int* s_rpre = s_psum + R + NW;                         // [ncols]
+        int* s_rtot = s_rpre + ncols;                          // [ncols]
+        int* s_any = s_rtot + ncols;                           // [num_blocks * EP_TOKENS_PER_BLOCK / 4] one byte a token
+        unsigned char* s_anyb = (unsigned char*)s_any;
+        const int ntok_all = a.num_blocks * EP_TOKENS_PER_BLOCK, n_all = a.num_blocks * nkeys;
+        for (int i = tid; i < 2 * ncols + ntok_all / 4; i += blockDim.x) s_rpre[i] = 0;
+        for (int i = tid; i < NW * (E + R); i += blockDim.x) s_we[i] = 0;
+        for (int i = tid; i < nkeys; i += blockDim.x) s_key[i] = s_rk[i] = -1;
+        __syncthreads();
+        if (key_total > 0) {
+            // (token and position of an id are carried along from load to load instead of divided out)
+            const int tok_step = EP_LAYOUT_THREADS / K, pos_step = EP_LAYOUT_THREADS - tok_step * K;
+            int tok = tid / K, pos = tid - tok * K;
+            // all ids at once, in up to three goes of eight a thread (as many as there are blocks to read: the same in
+            // every thread, so that a short launch neither asks for nor looks at the rest)
+            constexpr int GO = EP_RECOUNT_DEPTH / 3;
+            const int goes = (n_all + GO * EP_LAYOUT_THREADS - 1) / (GO * EP_LAYOUT_THREADS);      // 1..3 (the host's limit)
+            int64_t v[3][GO];
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                if (c >= goes) break;
+#pragma unroll
+                for (int u = 0; u < GO; ++u) v[c][u] = a.topk_idx[min((int64_t)tid + (c * GO + u) * EP_LAYOUT_THREADS, key_total - 1)];
+            }
+            __builtin_amdgcn_sched_barrier(0);      // (every id is asked for before the first is looked at)
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                if (c >= goes) break;
+#pragma unroll
+                for (int u = 0; u < GO; ++u) {
+                    const int i = tid + (c * GO + u) * EP_LAYOUT_THREADS;
+                    const bool valid = i < n_all && i < key_total && v[c][u] >= 0 && v[c][u] < a.num_experts;
+                    const int e = valid ? (int)v[c][u] : -1;
+                    if (valid) {
+                        atomicAdd(&s_rtot[e], 1);
+                        if (i < b * nkeys) atomicAdd(&s_rpre[e], 1);
+                        s_anyb[tok] = 1;
+                    }
+                    const int own = i - b * nkeys;
+                    if (own >= 0 && own < nkeys) {
+                        s_key[own] = (short)e;
+                        s_rk[own] = (short)(valid ? 0 : -1);
+                    }
+                    tok += tok_step;
+                    pos += pos_step;
+                    if (pos >= K) { pos -= K; ++tok; }
+                }
+            }
+        }
+        __syncthreads();
+        for (int t0 = 0; t0 < ntok_all; t0 += blockDim.x) {
+            const int t = t0 + tid;
+            const bool any = t < ntok_all && s_anyb[t] != 0;
+            const int all = __popcll(__ballot(any)), before = __popcll(__ballot(any && t < b * EP_TOKENS_PER_BLOCK));
+            if (lane == 0 && all > 0) {
+                atomicAdd(&s_rtot[El], all);
+                if (before > 0) atomicAdd(&s_rpre[El], before);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < EP_LAYOUT_MAX_COLS_PER_THREAD; ++k) {
+            const int c = tid + k * EP_LAYOUT_THREADS;
+            if (c >= ncols) continue;
+            pre[k] = s_rpre[c];
+            tot[k] = s_rtot[c];
+        }
+    }
+    // This workgroup's expert ids are asked for first (send side, up to four ids a thread).
     const bool folded = FOLD;
     const bool keys_early = folded && !RECV && nkeys <= 4 * EP_LAYOUT_THREADS && key_total > 0;
     // EP_LAYOUT_FOLDED: ep_layout_count has finished and left plain counts as 16-bit halves; the rows before this
@@ -435,7 +511,7 @@ __device__ __forceinline__ void layout_assign_body(const EpLayoutArgs& a) {
             s_key[i] = (short)e;
             s_rk[i] = (short)(e < 0 ? -1 : e / a.experts_per_rank);
         }
-    } else {
+    } else if (!recount) {            // (recounted: the ids are staged and the counters clear already)
         clear_counters();
         layout_load_keys(a, s_key, s_rk, s_psum, num_rows, RECV, kb);
         if (FOLD) fold_loads(v_first, s0, min(g0, FG - 1));

@@ -151,6 +151,7 @@ unsigned combine_lds_cap(int num_topk, bool specialised, int num_row_blocks, int
     if (share <= 1024u) return 0;
     return std::min(64u * 1024u, share - 1024u);       // n of them fit a CU, n + 1 do not
 }
+std::atomic<int> g_recount_limit{2 * EP_RECOUNT_DEPTH};   // blocks x top-k up to which one partition's slot assignment counts all ids itself
 std::atomic<int> g_fold_max_blocks{256};    // up to this many layout workgroups the slot assignment sums the block counts itself
 
 std::string library_dir() {
@@ -291,10 +292,20 @@ void launch_layout(EpLayoutArgs& la, int num_blocks, void* stream) {
     //  the rows where its sums meet, take the scan kernel at any size)
     const bool fold = num_blocks <= g_fold_max_blocks and la.cnt_stride <= 8 * EP_LAYOUT_THREADS and
                       layout_assign_lds(E, R, K, la.cnt_stride) <= 64 * 1024;
-    la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE : (fold ? EP_LAYOUT_FOLDED : EP_LAYOUT_SCANNED);
-    const unsigned smem_assign = layout_assign_lds(E, R, K, la.scan_mode == EP_LAYOUT_FOLDED ? la.cnt_stride : 0);
+    // a few blocks of one partition (send side): the slot assignment counts the ids of all blocks itself, a launch less
+    // (two histograms of El + R ints and a byte a token on top of its LDS)
+    const unsigned recount_extra = (unsigned)(2 * (E / R + R)) * sizeof(int) + (unsigned)num_blocks * EP_TOKENS_PER_BLOCK;
+    const bool recount = R == 1 and not la.recv_mode and not la.send_only and num_blocks >= 2 and
+                         (int64_t)num_blocks * K <= std::min(g_recount_limit.load(), 2 * EP_RECOUNT_DEPTH) and
+                         layout_assign_lds(E, R, K, 0) + recount_extra <= 64 * 1024;
+    la.scan_mode = num_blocks == 1 ? EP_LAYOUT_SINGLE
+                   : recount       ? EP_LAYOUT_RECOUNTED
+                   : fold          ? EP_LAYOUT_FOLDED
+                                   : EP_LAYOUT_SCANNED;
+    const unsigned smem_assign = layout_assign_lds(E, R, K, la.scan_mode == EP_LAYOUT_FOLDED ? la.cnt_stride : 0) +
+                                 (la.scan_mode == EP_LAYOUT_RECOUNTED ? recount_extra : 0u);
     EP_HOST_ASSERT(smem_assign <= 64 * 1024);
-    if (la.scan_mode != EP_LAYOUT_SINGLE)
+    if (la.scan_mode == EP_LAYOUT_FOLDED or la.scan_mode == EP_LAYOUT_SCANNED)
         launch(g_k.layout_count, num_blocks, EP_LAYOUT_THREADS, layout_count_lds(E, R, K), stream, la);
     if (la.scan_mode == EP_LAYOUT_SCANNED)
         launch(g_k.layout_scan, (unsigned)ceil_div(la.cnt_stride, 16), EP_SCAN_THREADS, 0, stream, la);
@@ -789,6 +800,8 @@ int64_t ep_dispatch_stamp(ep_buffer_t* b) {
 }
 
 void ep_set_layout_fold_max_blocks(int num_blocks) { g_fold_max_blocks = num_blocks; }
+
+void ep_set_layout_recount_limit(int blocks_times_topk) { g_recount_limit = blocks_times_topk; }
 
 void ep_set_combine_blocks_per_cu(int num_blocks) { g_combine_blocks_per_cu = num_blocks; }
 

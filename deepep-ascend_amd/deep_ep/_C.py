@@ -114,6 +114,7 @@ _ep_dispatch_epi = _sig('ep_dispatch_epilogue_launch', ctypes.c_int, ctypes.c_vo
                         ctypes.POINTER(_DispatchEpilogueArgs))
 _ep_stamp = _sig('ep_dispatch_stamp', ctypes.c_int64, ctypes.c_void_p)
 _ep_set_fold = _sig('ep_set_layout_fold_max_blocks', None, ctypes.c_int)
+_ep_set_recount = _sig('ep_set_layout_recount_limit', None, ctypes.c_int)
 _ep_set_combine_cap = _sig('ep_set_combine_blocks_per_cu', None, ctypes.c_int)
 _ep_dispatch_static = _sig('ep_dispatch_static_launch', ctypes.c_int, ctypes.POINTER(_DispatchArgs),
                            ctypes.POINTER(_DispatchEpilogueArgs))
@@ -274,6 +275,12 @@ def set_layout_fold_max_blocks(num_blocks: int) -> None:
     """Tuning: up to this many layout workgroups (128 tokens each) the slot-assignment kernel sums the
     per-workgroup histograms itself; beyond, a scan kernel runs in between.  Results do not depend on it."""
     _ep_set_fold(int(num_blocks))
+
+
+def set_layout_recount_limit(blocks_times_topk: int) -> None:
+    """Tuning: with one partition and few layout blocks (blocks x top-k up to this limit, at most 48; 0: never) the slot
+    assignment counts the ids of all blocks itself and the histogram kernel is not launched.  Results do not depend on it."""
+    _ep_set_recount(int(blocks_times_topk))
 
 
 class EventHandle:

@@ -172,6 +172,11 @@ int64_t ep_dispatch_stamp(ep_buffer_t* buf);
  * not depend on it. */
 void ep_set_layout_fold_max_blocks(int num_blocks);
 
+/* Tuning: with one partition and few layout blocks (blocks x top-k up to this limit; default and most 48, 0 turns it
+ * off) the histogram kernel is not launched: every workgroup of the slot assignment counts the ids of all blocks itself.
+ * Results do not depend on it. */
+void ep_set_layout_recount_limit(int blocks_times_topk);
+
 /* Tuning: workgroups (of 4 waves) of the single-partition combine kernel that a compute unit holds at once;
  * 0 lifts the cap, a negative value lets the library choose by top-k (the default: 3 at top-6 and top-8,
  * 4 at top-4, none at top-2 and for launches too small to fill the machine twice).  The cap is enforced through

@@ -256,27 +256,32 @@ def test_block_counts_at_their_16_bit_bound():
     buf.destroy()
 
 
-@pytest.mark.parametrize('T,E,K,R,rank', [(1500, 256, 8, 1, 0), (700, 64, 6, 4, 1)])
-def test_folded_and_scanned_block_prefixes_agree(T, E, K, R, rank):
-    """Several layout workgroups: the slot assignment either sums the histograms of the workgroups before it
-    itself, or reads the prefixes a scan kernel left.  Same handle tensors either way."""
+@pytest.mark.parametrize('T,E,K,R,rank', [(1500, 256, 8, 1, 0), (700, 64, 6, 4, 1), (700, 64, 6, 1, 0), (257, 256, 8, 1, 0),
+                                         (1000, 2048, 2, 1, 0)])
+def test_layout_paths_agree(T, E, K, R, rank):
+    """Several layout workgroups, four ways to the counts of the workgroups before one: the slot assignment sums the
+    histograms itself, or reads the prefixes a scan kernel left, or (one partition, few blocks: the last three shapes) no
+    histogram kernel runs and it counts the ids of all blocks itself.  Same handle tensors every way."""
     import deep_ep
     H, A = 128, 16
     topk, w = make_routing(T, E, K, seed=T + 1, masked=0.1)
     lay = O.rank_share_layout(topk.numpy(), E, R, rank, A, T)
     try:
-        for fold_max in (256, 1):                        # 1: every multi-block layout takes the scan kernel
+        # fold_max 1: every multi-block layout takes the scan kernel; recount limit 0: the histogram kernel always runs
+        for fold_max, recount in ((256, 48), (256, 0), (1, 0)):
             deep_ep._C.set_layout_fold_max_blocks(fold_max)
+            deep_ep._C.set_layout_recount_limit(recount)
             buf = _buffer(T, H, K, R, rank)
             _, _, _, handle, _ = buf.dispatch(make_tokens(T, H).to(DEV), topk_idx=topk.to(DEV), topk_weights=w.to(DEV),
                                               num_experts=E, expert_alignment=A, do_expand=True)
             torch.cuda.synchronize()
             for name in ('psum_num_recv_tokens_per_rank', 'psum_num_recv_tokens_per_expert',
                          'num_unaligned_recv_tokens_per_expert', 'dst_buffer_slot_idx', 'recv_src_metadata'):
-                assert np.array_equal(getattr(handle, name).cpu().numpy(), lay[name]), (fold_max, name)
+                assert np.array_equal(getattr(handle, name).cpu().numpy(), lay[name]), (fold_max, recount, name)
             buf.destroy()
     finally:
         deep_ep._C.set_layout_fold_max_blocks(256)
+        deep_ep._C.set_layout_recount_limit(48)
 
 
 @pytest.mark.parametrize('fused', [False, True])
