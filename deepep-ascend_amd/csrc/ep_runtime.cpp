@@ -290,8 +290,10 @@ void launch_layout(EpLayoutArgs& la, int num_blocks, void* stream) {
     const int E = la.num_experts, R = la.num_ranks, K = la.num_topk;
     // (the few shapes with more count columns than the summing instance has threads for, or whose LDS would not hold
     //  the rows where its sums meet, take the scan kernel at any size)
-    const bool fold = num_blocks <= g_fold_max_blocks and la.cnt_stride <= 8 * EP_LAYOUT_THREADS and
-                      layout_assign_lds(E, R, K, la.cnt_stride) <= 64 * 1024;
+    // (what the summing costs is rows a thread: blocks x column groups of 8 / threads.  The limit is quoted in blocks at
+    //  the headline's 264 columns, 33 groups; narrower rows, as the 40 columns of an EP32 partition, sum that many more)
+    const bool fold = (int64_t)num_blocks * (la.cnt_stride / 8) <= (int64_t)g_fold_max_blocks * 33 and
+                      la.cnt_stride <= 8 * EP_LAYOUT_THREADS and layout_assign_lds(E, R, K, la.cnt_stride) <= 64 * 1024;
     // a few blocks of one partition (send side): the slot assignment counts the ids of all blocks itself, a launch less
     // (two histograms of El + R ints and a byte a token on top of its LDS)
     const unsigned recount_extra = (unsigned)(2 * (E / R + R)) * sizeof(int) + (unsigned)num_blocks * EP_TOKENS_PER_BLOCK;

@@ -168,7 +168,8 @@ typedef struct ep_dispatch_recv_args {
 int64_t ep_dispatch_stamp(ep_buffer_t* buf);
 
 /* Tuning: number of layout workgroups (128 tokens each) up to which the slot-assignment kernel sums the
- * per-workgroup histograms itself instead of a scan kernel running in between (default 256).  Results do
+ * per-workgroup histograms itself instead of a scan kernel running in between (default 256; quoted for count rows of
+ * 264 columns, 256 local experts + one partition: with narrower rows the limit grows in proportion).  Results do
  * not depend on it. */
 void ep_set_layout_fold_max_blocks(int num_blocks);
 

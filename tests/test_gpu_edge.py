@@ -257,18 +257,19 @@ def test_block_counts_at_their_16_bit_bound():
 
 
 @pytest.mark.parametrize('T,E,K,R,rank', [(1500, 256, 8, 1, 0), (700, 64, 6, 4, 1), (700, 64, 6, 1, 0), (257, 256, 8, 1, 0),
-                                         (1000, 2048, 2, 1, 0)])
+                                         (1000, 2048, 2, 1, 0), (40000, 64, 2, 8, 3)])
 def test_layout_paths_agree(T, E, K, R, rank):
     """Several layout workgroups, four ways to the counts of the workgroups before one: the slot assignment sums the
     histograms itself, or reads the prefixes a scan kernel left, or (one partition, few blocks: the last three shapes) no
-    histogram kernel runs and it counts the ids of all blocks itself.  Same handle tensors every way."""
+    histogram kernel runs and it counts the ids of all blocks itself.  Same handle tensors every way.  (The last shape:
+    313 blocks of a partition with 16 count columns, which the slot assignment still sums itself.)"""
     import deep_ep
     H, A = 128, 16
     topk, w = make_routing(T, E, K, seed=T + 1, masked=0.1)
     lay = O.rank_share_layout(topk.numpy(), E, R, rank, A, T)
     try:
-        # fold_max 1: every multi-block layout takes the scan kernel; recount limit 0: the histogram kernel always runs
-        for fold_max, recount in ((256, 48), (256, 0), (1, 0)):
+        # fold_max 0: every multi-block layout takes the scan kernel; recount limit 0: the histogram kernel always runs
+        for fold_max, recount in ((256, 48), (256, 0), (0, 0)):
             deep_ep._C.set_layout_fold_max_blocks(fold_max)
             deep_ep._C.set_layout_recount_limit(recount)
             buf = _buffer(T, H, K, R, rank)
